@@ -1,0 +1,57 @@
+"""Builds the native parts in-tree: libi6fbw.so (HIP kernels + C ABI, hipcc, gfx950) and the
+PyTorch-ROCm binding fbw_core (links libi6fbw.so).  Takes the place of the reference's
+setup.py FBW entry (setup.py:29-33) and its import-time JIT fallback (fbw/__init__.py:10-24):
+nothing is compiled at import time, and nothing is hipified."""
+import os
+import subprocess
+import sys
+import sysconfig
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG, "csrc")
+OUT = os.path.join(PKG, "fbw")
+LIB = os.path.join(OUT, "libi6fbw.so")
+EXT = os.path.join(OUT, "fbw_core" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# packed-fp32 code generation is switched off for all device code
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def build_lib():
+    _run([HIPCC, *HIP_FLAGS, "-shared", os.path.join(CSRC, "fbw_kernels.hip"), "-o", LIB])
+    return LIB
+
+
+def build_ext():
+    import torch
+    from torch.utils import cpp_extension
+    inc = cpp_extension.include_paths()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=fbw_core", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I" + sysconfig.get_paths()["include"], "-I/opt/rocm/include"]
+    cmd += ["-I" + p for p in inc]
+    cmd += [os.path.join(CSRC, "fbw_torch.cpp"), "-o", EXT,
+            "-L" + OUT, "-li6fbw", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+            "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
+            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-Wl,-rpath,/opt/rocm/lib", "-Wno-attributes"]
+    _run(cmd)
+    return EXT
+
+
+def build_all():
+    build_lib()
+    build_ext()
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,91 @@
+"""ctypes view of libi6fbw.so, the C ABI declared in include/i6fbw.h.
+
+Used by the benchmark and the parity tests to call the library exactly as a foreign binding
+would: raw device pointers and sizes, caller-owned workspace, caller-chosen stream.  The
+PyTorch extension ``fbw_core`` links the same library directly.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "fbw", "libi6fbw.so")
+
+OUT_NEG_LOG = 0
+OUT_PROB = 1
+N_STAGES = 4
+STAGE_NAMES = ("prepare", "gather", "recurse", "combine")
+
+# every symbol include/i6fbw.h declares
+SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
+           "i6fbw_profile_enable", "i6fbw_profile_read")
+
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is not built; run `python -m i6_native_ops_amd.build`")
+        lib = ctypes.CDLL(LIB_PATH)
+        c = ctypes
+        lib.i6fbw_workspace_size.argtypes = [c.c_int] * 5 + [c.POINTER(c.c_size_t)]
+        lib.i6fbw_workspace_size.restype = c.c_int
+        lib.i6fbw_run.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_int64, c.c_void_p, c.c_void_p,
+                                  c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
+                                  c.c_void_p, c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
+        lib.i6fbw_run.restype = c.c_int
+        lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
+        lib.i6fbw_read_status.restype = c.c_int
+        lib.i6fbw_strerror.argtypes = [c.c_int]
+        lib.i6fbw_strerror.restype = c.c_char_p
+        lib.i6fbw_last_hip_error.restype = c.c_char_p
+        lib.i6fbw_profile_enable.argtypes = [c.c_int]
+        lib.i6fbw_profile_enable.restype = None
+        lib.i6fbw_profile_read.argtypes = [c.POINTER(c.c_float)]
+        lib.i6fbw_profile_read.restype = c.c_int
+        _lib = lib
+    return _lib
+
+
+class FbwError(RuntimeError):
+    def __init__(self, code, seq=None):
+        self.code = code
+        self.seq = seq
+        where = f" (sequence {seq})" if seq is not None and seq >= 0 else ""
+        super().__init__(f"i6fbw: {load().i6fbw_strerror(code).decode()}{where}")
+
+
+def workspace_size(T, B, F, E, n_states) -> int:
+    n = ctypes.c_size_t(0)
+    rc = load().i6fbw_workspace_size(T, B, F, E, n_states, ctypes.byref(n))
+    if rc != 0:
+        raise FbwError(rc)
+    return int(n.value)
+
+
+def run(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr, se_row_stride,
+        seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, sum_ptr, ws_ptr, ws_bytes, stream=0) -> None:
+    rc = load().i6fbw_run(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr,
+                          se_row_stride, seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, sum_ptr, ws_ptr,
+                          ws_bytes, stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def read_status(ws_ptr, B, stream=0):
+    code, seq = ctypes.c_int(0), ctypes.c_int(-1)
+    rc = load().i6fbw_read_status(ws_ptr, B, stream, ctypes.byref(code), ctypes.byref(seq))
+    if rc != 0:
+        raise FbwError(rc)
+    return int(code.value), int(seq.value)
+
+
+def profile_enable(on: bool) -> None:
+    load().i6fbw_profile_enable(1 if on else 0)
+
+
+def profile_read():
+    arr = (ctypes.c_float * N_STAGES)()
+    n = load().i6fbw_profile_read(arr)
+    return n, [float(x) for x in arr]

@@ -1,0 +1,113 @@
+// PyTorch-ROCm binding of libi6fbw.so: module `fbw_core` with the reference's interface
+// (i6_native_ops/fbw/fbw_torch.cpp:15-40): fbw(am_scores, edges, weights, start_end_states,
+// seq_lens, num_states, debug_options=DebugOptions()) -> [out (T,B,F), sum_output (T,B)].
+// torch is used for device memory and the current stream only; all arithmetic is behind the
+// C ABI declared in include/i6fbw.h.
+#include <cstdlib>
+#include <vector>
+
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include "../../include/i6fbw.h"
+
+namespace py = pybind11;
+
+// Same fields and defaults as the reference's DebugOptions.h:4-9.
+struct DebugOptions {
+    bool dump_alignment = false;
+    bool dump_output = false;
+    unsigned dump_every = 40u;
+    float pruning = 10.f;
+};
+
+// Same checks and messages as CHECK_INPUT (common/returnn_definitions.h:93-99).
+#define CHECK_CUDA(x) TORCH_CHECK(x.device().is_cuda(), #x " must be a CUDA tensor")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
+#define CHECK_TYPE(x, type) \
+    TORCH_CHECK(x.dtype() == type, "Expected " #x " to contain elements of type ", type, ", but got type ", x.dtype())
+#define CHECK_INPUT(x, type) \
+    CHECK_CUDA(x);           \
+    CHECK_CONTIGUOUS(x);     \
+    CHECK_TYPE(x, type)
+
+static bool status_check_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("I6FBW_ASYNC");
+        return !(e && e[0] == '1');
+    }();
+    return on;
+}
+
+static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
+                                      torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
+                                      int out_mode) {
+    CHECK_INPUT(am_scores, torch::kFloat32);
+    CHECK_INPUT(edges, torch::kInt32);
+    CHECK_INPUT(weights, torch::kFloat32);
+    CHECK_INPUT(start_end_states, torch::kInt32);
+    CHECK_INPUT(seq_lens, torch::kInt32);
+    // shape relations the reference asserts (fbw_op.cu:234-241,278-279)
+    TORCH_CHECK(am_scores.dim() == 3, "am_scores must have shape (T, B, F)");
+    TORCH_CHECK(edges.dim() == 2 && edges.size(0) == 4, "edges must have shape (4, E)");
+    TORCH_CHECK(weights.dim() == 1 && weights.size(0) == edges.size(1), "weights must have shape (E,)");
+    TORCH_CHECK(start_end_states.dim() == 2 && start_end_states.size(0) == 2 &&
+                    start_end_states.size(1) == am_scores.size(1),
+                "start_end_states must have shape (2, B)");
+    TORCH_CHECK(seq_lens.dim() == 1 && seq_lens.size(0) == am_scores.size(1), "seq_lens must have shape (B,)");
+    TORCH_CHECK(am_scores.size(0) > 0 && am_scores.size(1) > 0 && am_scores.size(2) > 0 && num_states > 0,
+                "NativeOp assertion failed: n_frames > 0, n_states > 0");
+    const int T = (int)am_scores.size(0), B = (int)am_scores.size(1), F = (int)am_scores.size(2);
+    const int E = (int)edges.size(1);
+
+    const c10::hip::HIPGuard guard(am_scores.device());
+    auto opts = torch::TensorOptions().device(am_scores.device());
+    torch::Tensor out = torch::empty_like(am_scores);
+    torch::Tensor sum_output = torch::empty({T, B}, opts.dtype(torch::kFloat32));
+    size_t ws_bytes = 0;
+    int rc = i6fbw_workspace_size(T, B, F, E, (int)num_states, &ws_bytes);
+    TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc));
+    torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, opts.dtype(torch::kUInt8));
+    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    rc = i6fbw_run(am_scores.data_ptr<float>(), am_scores.stride(0), am_scores.stride(1), edges.data_ptr<int32_t>(),
+                   edges.stride(0), weights.data_ptr<float>(), start_end_states.data_ptr<int32_t>(),
+                   start_end_states.stride(0), seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode,
+                   out.data_ptr<float>(), sum_output.data_ptr<float>(), workspace.data_ptr(), ws_bytes, (void*)stream);
+    TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
+    if (status_check_enabled()) {
+        int code = 0, seq = -1;
+        rc = i6fbw_read_status(workspace.data_ptr(), B, (void*)stream, &code, &seq);
+        TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
+        TORCH_CHECK(code == I6FBW_OK, "NativeOp: fbw: sequence ", seq, ": ", i6fbw_strerror(code));
+    }
+    return {out, sum_output};
+}
+
+std::vector<torch::Tensor> fbw(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
+                               torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
+                               DebugOptions debug_options = DebugOptions()) {
+    (void)debug_options;
+    return run(am_scores, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_NEG_LOG);
+}
+
+std::vector<torch::Tensor> fbw_posterior(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
+                                         torch::Tensor& start_end_states, torch::Tensor& seq_lens,
+                                         unsigned num_states) {
+    return run(am_scores, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_PROB);
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    py::class_<DebugOptions>(m, "DebugOptions")
+        .def(py::init<>())
+        .def_readwrite("dump_alignment", &DebugOptions::dump_alignment)
+        .def_readwrite("dump_output", &DebugOptions::dump_output)
+        .def_readwrite("dump_every", &DebugOptions::dump_every)
+        .def_readwrite("pruning", &DebugOptions::pruning);
+
+    m.def("fbw", &fbw, "Fast Baum-Welch routine (MI355X)", py::arg("am_scores"), py::arg("edges"), py::arg("weights"),
+          py::arg("start_end_states"), py::arg("seq_lens"), py::arg("num_states"),
+          py::arg("debug_options") = DebugOptions());
+    m.def("fbw_posterior", &fbw_posterior,
+          "Same as fbw but the first result holds the posteriors themselves (exp(-out)) with 0 in the holes");
+}

@@ -1,0 +1,113 @@
+/*
+ * C ABI of the MI355X (gfx950) full-sum forward-backward (FBW) library, libi6fbw.so.
+ *
+ * The reference has no C-level interface for this path; its only boundary is
+ * the pybind11 function `fbw_core.fbw` (i6_native_ops/fbw/fbw_torch.cpp:15-32)
+ * over the CUDA driver `fbw_cuda` (i6_native_ops/fbw/fbw_op.cu:226-393).  The
+ * entry points below are what a binding for that function needs: plain
+ * pointers and sizes, no torch types.  All data pointers are DEVICE pointers
+ * owned by the caller; the library never allocates or frees device memory and
+ * never synchronises the device (i6fbw_read_status excepted).
+ */
+#ifndef I6FBW_H
+#define I6FBW_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes (return values and i6fbw_read_status). */
+enum {
+    I6FBW_OK = 0,
+    I6FBW_ERR_INVALID_ARGUMENT = -1,   /* null pointer, non-positive T/B/F/n_states, bad out_mode */
+    I6FBW_ERR_WORKSPACE_TOO_SMALL = -2,
+    I6FBW_ERR_LAUNCH = -3,             /* a HIP launch failed; see i6fbw_last_hip_error() */
+    I6FBW_ERR_F_TOO_LARGE = -4,        /* F beyond what the row image / emission bitmap hold */
+    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* device-side: one sequence has more edges than supported */
+    I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* device-side: state ids of one sequence span more than 2*edges+2 */
+    I6FBW_ERR_SEQ_DEGREE = -12,           /* device-side: a state has more in- or out-edges than supported */
+    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side: states / distinct emissions of one sequence exceed LDS */
+    I6FBW_ERR_BAD_INDEX = -14             /* device-side: sequence, emission or state index out of range */
+};
+
+/* Layout of the posterior tensor written by i6fbw_run. */
+enum {
+    I6FBW_OUT_NEG_LOG = 0,   /* -log posterior, +inf where nothing contributes: what fbw_core.fbw returns
+                                (fbw_op.cu:366-377,392) */
+    I6FBW_OUT_PROB = 1       /* posterior itself, 0 where nothing contributes: what
+                                FastBaumWelchLoss.backward derives from it (fbw/__init__.py:40-44) */
+};
+
+/*
+ * Bytes of device workspace i6fbw_run needs for a problem of this size.
+ * Replaces the three raw cudaMalloc'ed buffers of fbw_op.cu:283-286.
+ */
+int i6fbw_workspace_size(int T, int B, int F, int E, int n_states, size_t* bytes);
+
+/*
+ * One FBW loss+posterior evaluation; replaces fbw_cuda (fbw_op.cu:226-393)
+ * as called from fbw (fbw_torch.cpp:15-29).
+ *
+ *   am_scores   float [T,B,F], -log probabilities, element strides am_stride_t / am_stride_b,
+ *               innermost stride 1                                   (fbw_op.cu:258,268-276)
+ *   edges       int32 [4,E] rows from, to, emission_idx, sequence_idx, row stride edge_row_stride
+ *                                                                    (fbw_op.cu:249-256)
+ *   weights     float [E], -log space                                (fbw_op.cu:257)
+ *   start_end   int32 [2,B] row 0 start states, row 1 end states, row stride se_row_stride
+ *                                                                    (fbw_op.cu:260-263)
+ *   seq_lens    int32 [B]                                            (fbw_op.cu:264)
+ *   n_states    number of states of the batch automaton              (fbw_torch.cpp:17)
+ *   out         float [T,B,F] contiguous, written completely         (fbw_op.cu:231,265)
+ *   sum_output  float [T,B] contiguous: total -log likelihood of sequence b in every frame
+ *               t < seq_lens[b], 0 elsewhere                         (fbw_op.cu:104-135,232)
+ *   workspace   device buffer of at least i6fbw_workspace_size bytes, 256-byte aligned
+ *   stream      hipStream_t to enqueue on (NULL = default stream); the call is asynchronous
+ *
+ * Returns I6FBW_OK or a negative host-side status.  Problems only the device can
+ * see (index out of range, an automaton beyond the supported size) are recorded in
+ * the workspace and reported by i6fbw_read_status; the affected sequences get NaN
+ * in out and sum_output.
+ */
+int i6fbw_run(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
+              const int32_t* edges, int64_t edge_row_stride,
+              const float* weights,
+              const int32_t* start_end, int64_t se_row_stride,
+              const int32_t* seq_lens,
+              int T, int B, int F, int E, int n_states, int out_mode,
+              float* out, float* sum_output,
+              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Waits for `stream` and copies the device-side status of the last i6fbw_run that
+ * used this workspace with batch size B: *code is I6FBW_OK or one of the device-side codes, *seq
+ * the first sequence it was seen on.  Replaces the reference's abort()/assert
+ * paths (fbw_op.cu:287-290, returnn_definitions.h:114-123) with a status.
+ */
+int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq);
+
+/* Text for a status code. */
+const char* i6fbw_strerror(int code);
+
+/* hipGetErrorString of the last failed HIP call of this thread ("" if none). */
+const char* i6fbw_last_hip_error(void);
+
+/*
+ * Average device time in milliseconds of each pipeline stage over all i6fbw_run
+ * calls since the last reset, measured with HIP events on the stream the kernels
+ * ran on.  Stage timing is off by default; i6fbw_profile_enable(1) turns it on
+ * (it adds event records between stages), i6fbw_profile_enable(0) turns it off
+ * and clears the sums.  stage_ms has room for I6FBW_N_STAGES entries:
+ * 0 edge preparation, 1 emission gather, 2 alpha/beta recursion, 3 combine + dense write.
+ * Waits for the recorded events.  Returns the number of calls averaged over.
+ */
+#define I6FBW_N_STAGES 4
+void i6fbw_profile_enable(int on);
+int i6fbw_profile_read(float* stage_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* I6FBW_H */

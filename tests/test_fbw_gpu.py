@@ -1,0 +1,71 @@
+"""Parity of the HIP path (through the C ABI of libi6fbw.so) with the CPU oracle.
+
+Bar (fp32 path): loss relative error <= 1e-5, posterior absolute error <= 1e-4.
+"""
+import numpy as np
+import pytest
+
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import brute_force, posterior, random_fsa, reference_fixture
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+POST_ATOL = 1e-4
+
+
+def check_against_oracle(oracle, args, threads=1):
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import run_cabi
+    am, edges, weights, start_end, seq_lens, n_states = args
+    want_out, want_loss = oracle.fbw_oracle(am, edges, weights, start_end, seq_lens, n_states, threads=threads)
+    want_post = posterior(want_out)
+    out, loss = run_cabi(*args, out_mode=cabi.OUT_NEG_LOG)
+    np.testing.assert_allclose(loss, want_loss, rtol=LOSS_RTOL, atol=1e-6)
+    assert (loss[want_loss == 0] == 0).all()
+    np.testing.assert_allclose(posterior(out), want_post, rtol=0, atol=POST_ATOL)
+    # holes are +inf in exactly the same places (a posterior below float range may differ)
+    assert (np.isposinf(out) | (want_post < 1e-30) == np.isposinf(want_out) | (want_post < 1e-30)).all()
+    prob, loss2 = run_cabi(*args, out_mode=cabi.OUT_PROB)
+    np.testing.assert_array_equal(loss2, loss)
+    np.testing.assert_allclose(prob, want_post, rtol=0, atol=POST_ATOL)
+    assert (prob[np.isposinf(want_out)] == 0).all()
+    return out, loss
+
+
+@pytest.mark.parametrize("seq_len", [5, 4, 1, 0, 6, -3])
+def test_reference_fixture(oracle, seq_len):
+    out, loss = check_against_oracle(oracle, reference_fixture(seq_len))
+    if seq_len == 5:   # closed form, test/fbw.py fixture
+        np.testing.assert_allclose(loss[:, 0], 5 - np.log(0.73224), rtol=2e-6)
+        np.testing.assert_allclose(posterior(out).sum(-1), 1.0, atol=1e-5)   # test/fbw.py:60-64
+
+
+@pytest.mark.parametrize("seed", range(25))
+def test_random_automata_brute_force(oracle, seed):
+    rng = np.random.default_rng(100 + seed)
+    args = random_fsa(rng, B=int(rng.integers(1, 5)), F=int(rng.integers(1, 6)), T=int(rng.integers(1, 8)))
+    out, loss = check_against_oracle(oracle, args)
+    want_loss, want_post = brute_force(*args)
+    np.testing.assert_allclose(loss, want_loss, rtol=LOSS_RTOL, atol=1e-5)
+    np.testing.assert_allclose(posterior(out), want_post, atol=POST_ATOL)
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("tiny", {}),
+    ("tiny", dict(shuffle_edges=True)),
+    ("monophone", dict(T=80, B=6, F=60)),
+    ("monophone", {}),
+    ("monophone", dict(shuffle_edges=True, seed=5)),
+    ("cart", dict(T=120, B=4, F=500)),
+    ("cart", dict(T=300, B=3, F=12001, shuffle_edges=True)),
+    ("ctc", dict(T=40, B=8, F=50)),
+    ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
+    ("longform", dict(T=200, B=2, F=300)),
+    ("longform", dict(T=1200, B=2, F=999, n_labels=(150, 200))),     # > 512 states: second size class
+    ("longform", dict(T=4000, B=1, F=777, n_labels=(700, 800))),     # > 2048 states: third size class
+])
+def test_workloads_small(oracle, name, kw):
+    W = make_workload(name, **kw)
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states),
+                         threads=8)
