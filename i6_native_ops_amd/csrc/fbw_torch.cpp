@@ -6,8 +6,8 @@
 #include <cstdlib>
 #include <vector>
 
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include "../../include/i6fbw.h"
@@ -61,7 +61,8 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
     const int T = (int)am_scores.size(0), B = (int)am_scores.size(1), F = (int)am_scores.size(2);
     const int E = (int)edges.size(1);
 
-    const c10::hip::HIPGuard guard(am_scores.device());
+    // PyTorch-ROCm presents HIP devices under the device type "cuda"
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(am_scores.device());
     auto opts = torch::TensorOptions().device(am_scores.device());
     torch::Tensor out = torch::empty_like(am_scores);
     torch::Tensor sum_output = torch::empty({T, B}, opts.dtype(torch::kFloat32));
@@ -69,7 +70,7 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
     int rc = i6fbw_workspace_size(T, B, F, E, (int)num_states, &ws_bytes);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc));
     torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, opts.dtype(torch::kUInt8));
-    hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
     rc = i6fbw_run(am_scores.data_ptr<float>(), am_scores.stride(0), am_scores.stride(1), edges.data_ptr<int32_t>(),
                    edges.stride(0), weights.data_ptr<float>(), start_end_states.data_ptr<int32_t>(),
                    start_end_states.stride(0), seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode,

@@ -1,0 +1,85 @@
+"""CPU-side checks of the drop-in boundary: the C ABI library loads and exports every symbol
+include/i6fbw.h declares, host-side argument validation, workspace sizing, and the binding's
+input checks (no GPU compute)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "i6fbw.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(i6fbw_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from i6_native_ops_amd import cabi
+    lib = cabi.load()
+    names = declared_symbols()
+    assert set(names) == set(cabi.SYMBOLS)
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_workspace_size_and_argument_validation():
+    from i6_native_ops_amd import cabi
+    n = cabi.workspace_size(1000, 32, 12001, 27000, 12000)
+    assert 100e6 < n < 2e9
+    assert cabi.workspace_size(50, 2, 10, 60, 32) < n
+    for bad in [(0, 1, 1, 1, 1), (1, 0, 1, 1, 1), (1, 1, 0, 1, 1), (1, 1, 1, -1, 1), (1, 1, 1, 1, 0)]:
+        with pytest.raises(cabi.FbwError):
+            cabi.workspace_size(*bad)
+    # null pointers are refused on the host before anything is launched
+    with pytest.raises(cabi.FbwError) as e:
+        cabi.run(0, 0, 0, 0, 0, 0, 0, 0, 0, 5, 1, 2, 3, 2, 0, 0, 0, 0, 0, 0)
+    assert e.value.code == -1
+    assert b"invalid" in cabi.load().i6fbw_strerror(-1)
+    assert cabi.load().i6fbw_strerror(-12) != cabi.load().i6fbw_strerror(-13)
+
+
+def test_extension_module_surface():
+    import i6_native_ops_amd.fbw as fbw
+    assert callable(fbw.fbw_loss) and issubclass(fbw.FastBaumWelchLoss, torch.autograd.Function)
+    d = fbw.core.DebugOptions()     # defaults of DebugOptions.h:4-9
+    assert (d.dump_alignment, d.dump_output, d.dump_every, d.pruning) == (False, False, 40, 10.0)
+    d.dump_every = 7
+    assert d.dump_every == 7
+
+
+def test_binding_rejects_bad_inputs_like_the_reference():
+    # CHECK_INPUT (returnn_definitions.h:93-99): device first, then contiguity, then dtype
+    import i6_native_ops_amd.fbw as fbw
+    am = torch.zeros(5, 1, 2)
+    edges = torch.zeros(4, 3, dtype=torch.int32)
+    w = torch.zeros(3)
+    se = torch.zeros(2, 1, dtype=torch.int32)
+    sl = torch.zeros(1, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="am_scores must be a CUDA tensor"):
+        fbw.core.fbw(am, edges, w, se, sl, 2)
+    with pytest.raises(RuntimeError, match="am_scores must be a CUDA tensor"):
+        fbw.core.fbw(am, edges, w, se, sl, 2, fbw.core.DebugOptions())
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        fbw.fbw_loss(torch.zeros(1, 5, 2, requires_grad=True), (2, edges, w, se), sl)
+
+
+def test_workload_generators_are_deterministic_and_well_formed():
+    import numpy as np
+    from i6_native_ops_amd.fbw.workloads import WORKLOADS, make_workload
+    for name in WORKLOADS:
+        a = make_workload(name, with_am=False)
+        b = make_workload(name, with_am=False)
+        np.testing.assert_array_equal(a.edges, b.edges)
+        np.testing.assert_array_equal(a.weights, b.weights)
+        assert a.edges.dtype == np.int32 and a.edges.shape[0] == 4
+        assert a.edges[:2].max() < a.n_states and a.edges[2].max() < a.F and a.edges[3].max() < a.B
+        assert (a.seq_lens >= 1).all() and (a.seq_lens <= a.T).all()
+        assert a.algorithmic_bytes() > 4 * a.T * a.B * a.F
+    w = make_workload("cart", with_am=False)
+    assert (w.T, w.B, w.F) == (1000, 32, 12001)
+    per_seq_states = np.diff(np.append(w.start_end_states[0], w.n_states))
+    assert per_seq_states.max() <= 451 and per_seq_states.min() >= 301

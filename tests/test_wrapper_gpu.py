@@ -1,0 +1,119 @@
+"""The Python front end on the GPU: a port of the reference's own test (test/fbw.py) plus the
+behaviours a drop-in has to keep (return shape, ignored grad_loss, fbw_core.fbw contract,
+status reporting)."""
+import numpy as np
+import pytest
+import torch
+
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import posterior, reference_fixture
+
+pytestmark = pytest.mark.gpu
+
+
+def _fixture_tensors(device="cuda"):
+    log_probs = (
+        torch.tensor([[0.9, 0.1], [0.9, 0.1], [0.4, 0.6], [0.1, 0.9], [0.1, 0.9]], device=device,
+                     dtype=torch.float32, requires_grad=True).unsqueeze(0).log()
+    )
+    edges = torch.tensor([[0, 0, 0, 0], [0, 1, 0, 0], [1, 1, 1, 0]], device=device,
+                         dtype=torch.int32).transpose(0, 1).contiguous()
+    weights = torch.tensor([1, 1, 1], device=device, dtype=torch.float32)
+    start_end_states = torch.tensor([[0], [1]], dtype=torch.int32, device=device)
+    seq_lens = torch.tensor([5], dtype=torch.int32, device=device)
+    return log_probs, (2, edges, weights, start_end_states), seq_lens
+
+
+def test_grad_like_reference_test():
+    """test/fbw.py:8-64: no device memory is lost over the call, and -grad sums to 1 per frame."""
+    from i6_native_ops_amd.fbw import fbw_loss
+    log_probs, fsa, seq_lens = _fixture_tensors()
+    log_probs.retain_grad()
+    fbw_loss(log_probs.detach(), fsa, seq_lens)       # warm the caching allocator
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    free_pre = torch.cuda.mem_get_info()[0]
+    loss = fbw_loss(log_probs, fsa, seq_lens)
+    torch.cuda.empty_cache()
+    free_post = torch.cuda.mem_get_info()[0]
+    # the only memory still held is what the call returned / saved for backward
+    held = loss.numel() * 4 + log_probs.numel() * 4 * 2
+    assert free_pre - free_post <= max(held, 8 << 20), "memory leak detected in FBW op"
+    assert loss.shape == (5, 1)                        # (T, B), not (B,)
+    np.testing.assert_allclose(loss.detach().cpu().numpy()[:, 0], 5 - np.log(0.73224), rtol=2e-6)
+    loss.sum().backward()
+    grad = log_probs.grad
+    assert torch.isclose(grad.sum(-1).neg(), torch.full(log_probs.shape[:2], 1.0, device="cuda")).all()
+
+
+def test_backward_ignores_grad_loss():
+    """fbw/__init__.py:40-44 returns the posteriors whatever grad_loss is."""
+    from i6_native_ops_amd.fbw import fbw_loss
+    grads = []
+    for scale in (1.0, 7.0):
+        log_probs, fsa, seq_lens = _fixture_tensors()
+        log_probs.retain_grad()
+        (fbw_loss(log_probs, fsa, seq_lens) * scale).sum().backward()
+        grads.append(log_probs.grad.clone())
+    assert torch.equal(grads[0], grads[1])
+
+
+def test_core_fbw_contract(oracle):
+    """fbw_core.fbw returns [out (T,B,F) in -log space with +inf holes, sum_output (T,B)]."""
+    from i6_native_ops_amd.fbw import core
+    W = make_workload("monophone", T=80, B=6, F=60, shuffle_edges=True)
+    dev = "cuda"
+    out, loss = core.fbw(torch.from_numpy(W.am_scores).to(dev), torch.from_numpy(W.edges).to(dev),
+                         torch.from_numpy(W.weights).to(dev), torch.from_numpy(W.start_end_states).to(dev),
+                         torch.from_numpy(W.seq_lens).to(dev), W.n_states, core.DebugOptions())
+    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens,
+                                            W.n_states)
+    assert out.shape == (W.T, W.B, W.F) and loss.shape == (W.T, W.B)
+    np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(posterior(out.cpu().numpy()), posterior(want_out), atol=1e-4)
+    tiny = posterior(want_out) < 1e-30      # a posterior below float range may be a hole on one side only
+    assert ((np.isposinf(out.cpu().numpy()) | tiny) == (np.isposinf(want_out) | tiny)).all()
+    # the autograd path yields the same numbers
+    from i6_native_ops_amd.fbw import FastBaumWelchLoss
+    am = torch.from_numpy(W.am_scores).to(dev).requires_grad_(True)
+    fsa = (W.n_states, torch.from_numpy(W.edges).to(dev), torch.from_numpy(W.weights).to(dev),
+           torch.from_numpy(W.start_end_states).to(dev))
+    l2 = FastBaumWelchLoss.apply(am, fsa, torch.from_numpy(W.seq_lens).to(dev))
+    l2.sum().backward()
+    assert torch.equal(l2, loss)
+    np.testing.assert_allclose(am.grad.cpu().numpy(), posterior(want_out), atol=1e-4)
+
+
+def test_non_contiguous_and_wrong_dtype_inputs_raise():
+    from i6_native_ops_amd.fbw import core
+    log_probs, (n, edges, weights, se), seq_lens = _fixture_tensors()
+    am = log_probs.detach().neg().transpose(0, 1).contiguous()
+    with pytest.raises(RuntimeError, match="edges must be contiguous"):
+        core.fbw(am, edges.t().contiguous().t(), weights, se, seq_lens, n)
+    with pytest.raises(RuntimeError, match="Expected seq_lens to contain elements of type"):
+        core.fbw(am, edges, weights, se, seq_lens.long(), n)
+    with pytest.raises(RuntimeError, match="Expected am_scores to contain elements of type"):
+        core.fbw(am.double(), edges, weights, se, seq_lens, n)
+
+
+def test_device_side_status_is_reported():
+    """Indices the reference would read out of bounds with, and automata beyond the supported
+    size, surface as RuntimeError instead of the reference's abort()/undefined behaviour."""
+    from i6_native_ops_amd.fbw import core
+    log_probs, (n, edges, weights, se), seq_lens = _fixture_tensors()
+    am = log_probs.detach().neg().transpose(0, 1).contiguous()
+    bad = edges.clone()
+    bad[2, 1] = 5                       # emission index >= F
+    with pytest.raises(RuntimeError, match="index out of range"):
+        core.fbw(am, bad, weights, se, seq_lens, n)
+    bad = edges.clone()
+    bad[3, 0] = 3                       # sequence index >= B
+    with pytest.raises(RuntimeError, match="index out of range"):
+        core.fbw(am, bad, weights, se, seq_lens, n)
+    # a state with 9 incoming edges
+    many = torch.tensor([[0] * 9, [1] * 9, [0] * 9, [0] * 9], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="more than 8 incoming or outgoing edges"):
+        core.fbw(am, many, torch.zeros(9, device="cuda"), se, seq_lens, n)
+    # the good input still works afterwards
+    out, loss = core.fbw(am, edges, weights, se, seq_lens, n)
+    assert torch.isfinite(loss).all()
