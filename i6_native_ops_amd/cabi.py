@@ -12,8 +12,8 @@ LIB_PATH = os.path.join(_HERE, "fbw", "libi6fbw.so")
 
 OUT_NEG_LOG = 0
 OUT_PROB = 1
-N_STAGES = 4
-STAGE_NAMES = ("prepare", "gather", "recurse", "combine")
+N_STAGES = 5
+STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",

@@ -23,6 +23,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "../../include/i6fbw.h"
 
 namespace {
@@ -30,14 +32,26 @@ namespace {
 constexpr int KMAX = 8;               // in-/out-degree held in registers by the recursion
 constexpr int EB_MAX = 8192;          // edges of one sequence (capacity of the LDS sort)
 constexpr int F_BITMAP_MAX = 131072;  // emission ids covered by the LDS presence bitmap
-constexpr int S_MAX = 4096;           // states of one sequence (largest recursion class)
+constexpr int S_MAX = 4096;           // states of one sequence
 constexpr int D_MAX = 4096;           // distinct emissions of one sequence
-constexpr int TG = 8;                 // frames per gather workgroup
+#ifndef I6_TG
+#define I6_TG 8
+#endif
+#ifndef I6_GATHER_BFAST
+#define I6_GATHER_BFAST 0
+#endif
+constexpr int TG = I6_TG;             // frames per gather workgroup
 constexpr int TC = 8;                 // frames per combine workgroup
 constexpr int RENORM = 8;             // frames between renormalisations of the state vector
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
+constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of the combine kernel
+constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup (plus one loader wave)
 constexpr unsigned NO_STATE = 0xFFFFu;
+constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
+// Scores are kept in units of log 2 inside the workspace (exp2/log2 are single instructions).
+constexpr float LOG2E = 1.44269504088896341f;
+constexpr float LN2 = 0.693147180559945309f;
 #define INF_F __builtin_inff()
 
 struct SeqMeta {
@@ -61,7 +75,7 @@ __host__ __device__ inline long long state_off(long long edge_begin, int b) { re
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 
 struct Layout {
-    size_t meta, ellA, ellB, crec, cbegin, demis, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sortflag, eidx, ellA, ellB, crec, cbegin, demis, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
 };
 
@@ -72,17 +86,19 @@ Layout make_layout(long long T, long long B, long long E) {
     l.ss_total = round16(2 * E) + 32 * B + 16;
     l.gg_total = round16(E) + 32 * B + 16;
     size_t o = 0;
-    l.meta = o;   o = align256(o + sizeof(SeqMeta) * B);
-    l.ellA = o;   o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
-    l.ellB = o;   o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
-    l.crec = o;   o = align256(o + sizeof(uint4) * (E + 1));
-    l.cbegin = o; o = align256(o + sizeof(int) * l.gg_total);
-    l.demis = o;  o = align256(o + sizeof(int) * l.gg_total);
-    l.offA = o;   o = align256(o + sizeof(double) * B * T);
-    l.offB = o;   o = align256(o + sizeof(double) * B * T);
-    l.alpha = o;  o = align256(o + sizeof(float) * l.ss_total * T);
-    l.beta = o;   o = align256(o + sizeof(float) * l.ss_total * T);
-    l.gtab = o;   o = align256(o + sizeof(float) * l.gg_total * T);
+    l.meta = o;     o = align256(o + sizeof(SeqMeta) * B);
+    l.sortflag = o; o = align256(o + sizeof(int) * (E / SCAN_BLOCK + 2));
+    l.eidx = o;     o = align256(o + sizeof(int) * (E + 1));
+    l.ellA = o;     o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
+    l.ellB = o;     o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
+    l.crec = o;     o = align256(o + sizeof(uint4) * (E + 1));
+    l.cbegin = o;   o = align256(o + sizeof(int) * l.gg_total);
+    l.demis = o;    o = align256(o + sizeof(int) * l.gg_total);
+    l.offA = o;     o = align256(o + sizeof(double) * B * T);
+    l.offB = o;     o = align256(o + sizeof(double) * B * T);
+    l.alpha = o;    o = align256(o + sizeof(float) * l.ss_total * T);
+    l.beta = o;     o = align256(o + sizeof(float) * l.ss_total * T);
+    l.gtab = o;     o = align256(o + sizeof(float) * l.gg_total * T);
     l.total = o;
     return l;
 }
@@ -96,25 +112,43 @@ __device__ inline int seq_error(const SeqMeta& m) { return m.err ? m.err : (m.er
 __device__ inline int rec_class(const SeqMeta& m) {
     if (seq_error(m)) return -1;
     if (m.L == 0 || m.n_edges == 0) return 0;
-    if (m.SP <= 512 && m.DP <= 512) return 1;
-    if (m.SP <= 2048 && m.DP <= 2048) return 2;
+    if (m.SP <= REC_THREADS && m.DP <= 512) return 1;
+    if (m.SP <= 4 * REC_THREADS && m.DP <= 2048) return 2;
     return 3;
 }
-// Combine class: 1 handles errors, empty sequences and sequences of up to 1024 edges.
-__device__ inline int comb_class(const SeqMeta& m) {
-    if (seq_error(m) || m.L == 0 || m.n_edges == 0) return 1;
-    return m.n_edges <= 1024 ? 1 : 2;
-}
 
-__device__ inline float wave_min(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
+// The frames [0, L) of a sequence are cut into nch chunks; chunk k covers [chunk_lo(k), chunk_lo(k+1)).
+__device__ __forceinline__ int chunk_lo(int L, int k, int nch) { return (int)((long long)k * L / nch); }
+
+// wave-wide minimum in lane 63 (DPP row operations, no LDS traffic)
+__device__ __forceinline__ float wave_min_dpp(float v) {
+#define I6_DPP_MIN(ctrl, rmask)                                                                          \
+    v = fminf(v, __uint_as_float((unsigned)__builtin_amdgcn_update_dpp((int)__float_as_uint(v), (int)__float_as_uint(v), \
+                                                                       ctrl, rmask, 0xf, false)))
+    I6_DPP_MIN(0x111, 0xf);   // row_shr:1
+    I6_DPP_MIN(0x112, 0xf);   // row_shr:2
+    I6_DPP_MIN(0x114, 0xf);   // row_shr:4
+    I6_DPP_MIN(0x118, 0xf);   // row_shr:8  -> lane 15 of each row holds the row minimum
+    I6_DPP_MIN(0x142, 0xa);   // row_bcast:15 into rows 1 and 3
+    I6_DPP_MIN(0x143, 0xc);   // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave minimum
+#undef I6_DPP_MIN
     return v;
 }
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+// wave-wide sum in lane 63, fixed association order
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+#define I6_DPP_ADD(ctrl, rmask)                                                                 \
+    v += __uint_as_float((unsigned)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), ctrl, rmask, 0xf, false))
+    I6_DPP_ADD(0x111, 0xf);
+    I6_DPP_ADD(0x112, 0xf);
+    I6_DPP_ADD(0x114, 0xf);
+    I6_DPP_ADD(0x118, 0xf);
+    I6_DPP_ADD(0x142, 0xa);
+    I6_DPP_ADD(0x143, 0xc);
+#undef I6_DPP_ADD
     return v;
+}
+__device__ __forceinline__ float lane63(float v) {
+    return __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)__float_as_uint(v), 63));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -126,8 +160,22 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
-    SeqMeta* meta; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis;
+    SeqMeta* meta; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis;
 };
+
+// sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never decrease
+__global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int E, int* sortflag) {
+    __shared__ int bad;
+    if (threadIdx.x == 0) bad = 0;
+    __syncthreads();
+    const int base = blockIdx.x * SCAN_BLOCK;
+    int mybad = 0;
+    for (int i = base + threadIdx.x; i < min(E - 1, base + SCAN_BLOCK); i += 256)
+        mybad |= (unsigned)e_seq[i] > (unsigned)e_seq[i + 1];
+    if (mybad) atomicOr(&bad, 1);
+    __syncthreads();
+    if (threadIdx.x == 0) sortflag[blockIdx.x] = !bad;
+}
 
 __device__ inline int block_excl_scan(int v, int* wsum, int nwaves, int* total) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -150,25 +198,38 @@ __device__ inline int block_excl_scan(int v, int* wsum, int nwaves, int* total) 
     return base + incl - v;
 }
 
-// first index i in [0,n) with (keys[i] >> 32) >= p
-__device__ inline int lower_bound_hi(const unsigned long long* keys, int n, unsigned p) {
+constexpr int KEY_POS_BITS = 13;   // EB_MAX = 2^13 positions; the primary key sits above them
+static_assert((1 << KEY_POS_BITS) == EB_MAX, "key layout");
+
+// first index i in [0,n) with (keys[i] >> KEY_POS_BITS) >= p
+__device__ inline int lower_bound_hi(const unsigned* keys, int n, unsigned p) {
     int lo = 0, hi = n;
     while (lo < hi) {
         int mid = (lo + hi) >> 1;
-        if ((unsigned)(keys[mid] >> 32) < p) lo = mid + 1; else hi = mid;
+        if ((keys[mid] >> KEY_POS_BITS) < p) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+// first index i in [0,n) with (unsigned)a[i] >= v, for a non-decreasing global array
+__device__ inline int lower_bound_u32(const int32_t* a, int n, unsigned v) {
+    int lo = 0, hi = n;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if ((unsigned)a[mid] < v) lo = mid + 1; else hi = mid;
     }
     return lo;
 }
 
 // grid (3, B): role 0 orders the edges of sequence b by target state (alpha), role 1 by source
 // state (beta), role 2 by emission slot (combine) and writes the shared part of the meta record.
+// Edge lists grouped by sequence (the usual case) are located by binary search; any other order
+// is handled by a stable scan over the whole list.
 __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
-    __shared__ unsigned long long keys[EB_MAX];
-    __shared__ int eidx[EB_MAX];
+    __shared__ unsigned keys[EB_MAX];
     __shared__ unsigned bitmap[F_BITMAP_MAX / 32];
     __shared__ int wordpfx[F_BITMAP_MAX / 32];
     __shared__ int wsum[16];
-    __shared__ int s_lt, s_bad, s_kmax;
+    __shared__ int s_lt, s_bad, s_kmax, s_sorted;
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -178,31 +239,52 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     const int32_t* e_seq = a.edges + 3 * a.edge_stride;
     const int E = a.E;
 
-    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_min = 0xffffffffu; s_max = 0u; }
+    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; }
     __syncthreads();
+    const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
+    int unsorted = 0;
+    for (int i = tid; i < nflag; i += 1024) unsorted |= !a.sortflag[i];
+    if (unsorted) atomicAnd(&s_sorted, 0);
+    __syncthreads();
+    const bool sorted = s_sorted != 0;
 
-    // pass 1: count the edges of earlier sequences and of this one, state range, index checks
+    int edge_begin, n_edges, pos = 0;
+    int bad = 0;
+    unsigned mn = 0xffffffffu, mx = 0u;
     const int chunk = (E + 1023) / 1024;
     const int lo = min(E, tid * chunk), hi = min(E, lo + chunk);
-    int lt = 0, eq = 0, bad = 0;
-    unsigned mn = 0xffffffffu, mx = 0u;
-    for (int i = lo; i < hi; i++) {
-        unsigned s = (unsigned)e_seq[i];
-        lt += s < (unsigned)b;
-        if (s == (unsigned)b) {
-            eq++;
+    if (sorted) {
+        edge_begin = lower_bound_u32(e_seq, E, (unsigned)b);
+        n_edges = lower_bound_u32(e_seq, E, (unsigned)b + 1u) - edge_begin;
+        if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B) bad = 1;
+        for (int i = edge_begin + tid; i < edge_begin + n_edges; i += 1024) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
             mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
             if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
         }
-        if (b == 0 && s >= (unsigned)a.B) bad = 1;
+        if (bad) atomicOr(&s_bad, 1);
+        if (mn <= mx) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
+        __syncthreads();
+    } else {
+        // count the edges of earlier sequences and of this one, state range, index checks
+        int lt = 0, eq = 0;
+        for (int i = lo; i < hi; i++) {
+            unsigned s = (unsigned)e_seq[i];
+            lt += s < (unsigned)b;
+            if (s == (unsigned)b) {
+                eq++;
+                unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
+                mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
+                if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
+            }
+            if (b == 0 && s >= (unsigned)a.B) bad = 1;
+        }
+        if (lt) atomicAdd(&s_lt, lt);
+        if (bad) atomicOr(&s_bad, 1);
+        if (eq) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
+        pos = block_excl_scan(eq, wsum, 16, &n_edges);   // barriers inside publish the atomics too
+        edge_begin = s_lt;
     }
-    if (lt) atomicAdd(&s_lt, lt);
-    if (bad) atomicOr(&s_bad, 1);
-    if (eq) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
-    int n_edges;
-    int pos = block_excl_scan(eq, wsum, 16, &n_edges);   // barriers inside publish the atomics too
-    const int edge_begin = s_lt;
 
     const unsigned st_state = (unsigned)a.start_end[b], en_state = (unsigned)a.start_end[a.se_stride + b];
     unsigned smin = min(min(s_min, st_state), en_state), smax = max(max(s_max, st_state), en_state);
@@ -218,17 +300,23 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     const int SP = (int)round16(S);
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
+    // i-th edge of this sequence in input order
+    int* eidx = a.eidx + edge_begin;
+    auto edge_at = [&](int i) -> int { return sorted ? edge_begin + i : eidx[i]; };
+
     int D = 0;
     if (!err && n_edges > 0) {
-        // pass 2: stable list of this sequence's edge indices
-        for (int i = lo; i < hi; i++)
-            if ((unsigned)e_seq[i] == (unsigned)b) eidx[pos++] = i;
+        if (!sorted) {
+            // stable list of this sequence's edge indices (every role writes the same values)
+            for (int i = lo; i < hi; i++)
+                if ((unsigned)e_seq[i] == (unsigned)b) eidx[pos++] = i;
+        }
         // emission presence bitmap -> slot = rank of the emission id among the distinct ones
         const int nwords = (a.F + 31) >> 5;
         for (int w = tid; w < nwords; w += 1024) bitmap[w] = 0u;
         __syncthreads();
         for (int i = tid; i < n_edges; i += 1024) {
-            unsigned em = (unsigned)e_emis[eidx[i]];
+            unsigned em = (unsigned)e_emis[edge_at(i)];
             atomicOr(&bitmap[em >> 5], 1u << (em & 31));
         }
         __syncthreads();
@@ -262,15 +350,15 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
         return (unsigned)wordpfx[em >> 5] + (unsigned)__popc(bitmap[em >> 5] & ((1u << (em & 31)) - 1u));
     };
 
-    // sort keys: (primary << 32) | stable position; ties keep the input order
+    // sort keys: (primary << 13) | position in input order; ties keep the input order
     int N = 2;
     while (N < n_edges) N <<= 1;
     for (int i = tid; i < N; i += 1024) {
-        unsigned long long k = ~0ull;
+        unsigned k = ~0u;
         if (i < n_edges) {
-            int e = eidx[i];
+            int e = edge_at(i);
             unsigned p = role == 0 ? (unsigned)e_to[e] - smin : role == 1 ? (unsigned)e_from[e] - smin : slot_of((unsigned)e_emis[e]);
-            k = ((unsigned long long)p << 32) | (unsigned)i;
+            k = (p << KEY_POS_BITS) | (unsigned)i;
         }
         keys[i] = k;
     }
@@ -280,7 +368,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
             for (int i = tid; i < N; i += 1024) {
                 int ixj = i ^ j;
                 if (ixj > i) {
-                    unsigned long long x = keys[i], y = keys[ixj];
+                    unsigned x = keys[i], y = keys[ixj];
                     bool up = (i & k) == 0;
                     if ((x > y) == up) { keys[i] = y; keys[ixj] = x; }
                 }
@@ -288,14 +376,16 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
             __syncthreads();
         }
     }
+    constexpr unsigned POS_MASK = (1u << KEY_POS_BITS) - 1u;
 
     if (role < 2) {
         // ELL table: entry (k, s) = k-th edge (in input order) entering (role 0) / leaving (role 1)
-        // local state s, as {other state | slot << 16, weight}; unused entries point at NO_STATE.
+        // local state s, as {other state | slot << 16, weight * log2(e)}; unused entries point at
+        // NO_STATE.
         uint2* ell = (role == 0 ? a.ellA : a.ellB) + (size_t)KMAX * soff;
         int kmax = 0;
         for (int i = tid; i < n_edges; i += 1024) {
-            unsigned p = (unsigned)(keys[i] >> 32);
+            unsigned p = keys[i] >> KEY_POS_BITS;
             kmax = max(kmax, i - lower_bound_hi(keys, n_edges, p) + 1);
         }
         if (kmax) atomicMax(&s_kmax, kmax);
@@ -310,20 +400,20 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
         for (int i = tid; i < K * SP; i += 1024) ell[i] = make_uint2(NO_STATE, 0u);
         __syncthreads();
         for (int i = tid; i < n_edges; i += 1024) {
-            unsigned p = (unsigned)(keys[i] >> 32);
+            unsigned p = keys[i] >> KEY_POS_BITS;
             int k = i - lower_bound_hi(keys, n_edges, p);
-            int e = eidx[(unsigned)keys[i]];
+            int e = edge_at((int)(keys[i] & POS_MASK));
             unsigned other = (role == 0 ? (unsigned)e_from[e] : (unsigned)e_to[e]) - smin;
             unsigned slot = slot_of((unsigned)e_emis[e]);
-            ell[(size_t)k * SP + p] = make_uint2(other | (slot << 16), __float_as_uint(a.weights[e]));
+            ell[(size_t)k * SP + p] = make_uint2(other | (slot << 16), __float_as_uint(a.weights[e] * LOG2E));
         }
     } else {
         // combine order: edges sorted by slot; CSR begin per slot; list of distinct emission ids
         uint4* crec = a.crec + edge_begin;
         for (int i = tid; i < n_edges; i += 1024) {
-            int e = eidx[(unsigned)keys[i]];
+            int e = edge_at((int)(keys[i] & POS_MASK));
             unsigned f = (unsigned)e_from[e] - smin, t = (unsigned)e_to[e] - smin;
-            crec[i] = make_uint4(f | (t << 16), __float_as_uint(a.weights[e]), (unsigned)(keys[i] >> 32), 0u);
+            crec[i] = make_uint4(f | (t << 16), __float_as_uint(a.weights[e] * LOG2E), keys[i] >> KEY_POS_BITS, 0u);
         }
         int* cb = a.cbegin + goff;
         for (int d = tid; d <= D; d += 1024) cb[d] = d == D ? n_edges : lower_bound_hi(keys, n_edges, (unsigned)d);
@@ -343,23 +433,28 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// stage 2: gather  gtab[b][t][slot] = am[t, b, demis[b][slot]]  for t < L_b
+// stage 2: gather  gtab[b][t][slot] = log2(e) * am[t, b, demis[b][slot]]  for t < L_b
 // ---------------------------------------------------------------------------------------------
 struct GatherArgs {
     const float* am; long long st_t, st_b;
     int T, B;
     const SeqMeta* meta; const int* demis; float* gtab;
+    int nch, k0, k1;     // this launch covers chunks k0 (blockIdx.z == 0) and k1 (blockIdx.z == 1)
 };
 
 __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
-    const int b = blockIdx.y, t0 = blockIdx.x * TG;
+    const int b = blockIdx.y;
     const SeqMeta m = a.meta[b];
-    if (rec_class(m) <= 0 || t0 >= m.L) return;
+    if (rec_class(m) <= 0) return;
+    const int k = blockIdx.z ? a.k1 : a.k0;
+    const int c0 = chunk_lo(m.L, k, a.nch), c1 = chunk_lo(m.L, k + 1, a.nch);
+    const int t0 = c0 + blockIdx.x * TG;
+    if (t0 >= c1) return;
     const long long goff = slot_off(m.edge_begin, b);
     const int* de = a.demis + goff;
     float* g = a.gtab + (size_t)a.T * goff;
     const float* am = a.am + (long long)b * a.st_b;
-    const int nt = min(TG, m.L - t0);
+    const int nt = min(TG, c1 - t0);
     for (int idx = threadIdx.x; idx < m.DP; idx += 256) {
         const int e = de[idx];
         float v[TG];
@@ -368,36 +463,99 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
             if (tt < nt) v[tt] = am[(long long)(t0 + tt) * a.st_t + e];
 #pragma unroll
         for (int tt = 0; tt < TG; tt++)
-            if (tt < nt) g[(size_t)(t0 + tt) * m.DP + idx] = v[tt];
+            if (tt < nt) g[(size_t)(t0 + tt) * m.DP + idx] = v[tt] * LOG2E;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // stage 3: recursion.  Workgroup 2b walks alpha of sequence b forward, workgroup 2b+1 walks beta
 // backward.  Rows stored for frame t: alpha_t (state vector before frame t is consumed) and
-// beta_{t+1} (after it), each relative to an offset kept in double precision.
+// beta_{t+1} (after it), in units of log 2, each relative to an offset kept in double precision.
 // ---------------------------------------------------------------------------------------------
 struct RecArgs {
     int T, B;
     const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab;
     float* alpha; float* beta; double* offA; double* offB;
+    int nch, launch;     // launch j advances alpha over chunk j and beta over chunk nch-1-j
 };
 
+// Steps [*s0, *s1) of direction dir that belong to launch `launch`.  Step i consumes frame i (alpha)
+// or L-1-i (beta); there are L-1 steps in all.
+__device__ __forceinline__ void step_range(int L, int dir, int nch, int launch, int* s0, int* s1) {
+    if (!dir) {
+        *s0 = chunk_lo(L, launch, nch);
+        *s1 = min(chunk_lo(L, launch + 1, nch), L - 1);
+    } else {
+        const int k = nch - 1 - launch;
+        *s0 = L - chunk_lo(L, k + 1, nch);
+        *s1 = L - max(chunk_lo(L, k, nch), 1);
+    }
+    if (*s1 < *s0) *s1 = *s0;
+}
+
 // Barrier for LDS traffic only: waits for this wave's LDS operations and not for its global
-// stores.  (On gfx9-family hardware loads and stores retire out of order with each other, so
-// a wave that has both in flight can only wait for "all of them"; the recursion therefore
-// keeps them in different waves: compute waves only store, the loader wave only loads.)
+// memory traffic (the compute waves' row stores, the loader wave's prefetches).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Compute waves: thread tid owns states tid + j*THREADS.  Per frame: read the predecessor
-// values and the staged emission scores from LDS, log-sum-exp in a fixed order, write the new
-// value to the other LDS buffer and to the workspace row, one barrier.
+struct RecCursor {
+    float* wp; long long wstep;      // workspace row written by the next step
+    double* op; int ostep;           // its offset
+    double c; bool pending;          // running offset, renormalisation requested by the last step
+};
+
+// One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
+// LDS, log-sum-exp (base 2) in a fixed order, result to the other LDS buffer and the workspace.
+template <int THREADS, int J, int KT>
+__device__ __forceinline__ void recurse_step(const int i, const int SP, const char* __restrict__ stc, float* __restrict__ stn,
+                                             const char* __restrict__ amc, float* __restrict__ wmin,
+                                             const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
+                                             const float (&ew)[J][KT], RecCursor& cur) {
+    constexpr int NW = THREADS / 64;
+    const int tid = threadIdx.x;
+    float pend = 0.f;
+    if (cur.pending) {
+        float mn = wmin[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) mn = fminf(mn, wmin[w]);
+        pend = mn == INF_F ? 0.f : mn;
+        cur.c += (double)pend;
+    }
+    float rmin = INF_F;
+#pragma unroll
+    for (int j = 0; j < J; j++) {
+        const int s = tid + j * THREADS;
+        float v[KT];
+        float mn = INF_F;
+#pragma unroll
+        for (int k = 0; k < KT; k++) {
+            v[k] = *(const float*)(stc + eo[j][k]) + (ew[j][k] + *(const float*)(amc + es[j][k]));
+            mn = fminf(mn, v[k]);
+        }
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f(mn - v[k]);
+        // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
+        const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
+        stn[s] = r;
+        if (s < SP) cur.wp[s] = r;
+        rmin = fminf(rmin, r);
+    }
+    if (tid == 0) *cur.op = cur.c;
+    cur.wp += cur.wstep; cur.op += cur.ostep;
+    cur.pending = (i % RENORM) == RENORM - 1;
+    if (cur.pending) {
+        rmin = wave_min_dpp(rmin);
+        if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
+    }
+    lds_barrier();
+}
+
 template <int THREADS, int J, int KT>
 __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
                                                 float* __restrict__ st0, float* __restrict__ st1,
                                                 const float* __restrict__ am0, const float* __restrict__ am1,
                                                 float* __restrict__ wmin) {
-    constexpr int SCAP = THREADS * J, NW = THREADS / 64;
+    constexpr int SCAP = THREADS * J;
     const int tid = threadIdx.x;
     const int L = m.L, SP = m.SP, T = a.T;
     const long long soff = state_off(m.edge_begin, b);
@@ -406,6 +564,7 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
     double* offs = (dir ? a.offB : a.offA) + (size_t)b * T;
     const int K = dir ? m.Kout : m.Kin;
 
+    // edges of my states -> registers, as LDS byte offsets of the other state / the emission slot
     unsigned eo[J][KT], es[J][KT];
     float ew[J][KT];
 #pragma unroll
@@ -417,73 +576,127 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
             if (k < K && s < SP) r = ell[(size_t)k * SP + s];
             unsigned other = r.x & 0xFFFFu;
             if (other == NO_STATE) other = SCAP;          // LDS cell that always holds +inf
-            eo[j][k] = other;
-            es[j][k] = r.x >> 16;
+            eo[j][k] = other * 4u;
+            es[j][k] = (r.x >> 16) * 4u;
             ew[j][k] = __uint_as_float(r.y);
         }
     }
 
+    // state before the first step of this launch: the initial vector, or the row an earlier
+    // launch stored (values relative to the offset stored beside it)
+    int s0, s1;
+    step_range(L, dir, a.nch, a.launch, &s0, &s1);
     const int init_state = dir ? m.end_local : m.start_local;
-    const int init_row = dir ? L - 1 : 0;
+    const int row0 = dir ? L - 1 - s0 : s0;
 #pragma unroll
     for (int j = 0; j < J; j++) {
         const int s = tid + j * THREADS;
-        const float v = s == init_state ? 0.f : INF_F;
+        float v;
+        if (s0 == 0) {
+            v = s == init_state ? 0.f : INF_F;
+            if (s < SP) ws[(size_t)row0 * SP + s] = v;
+        } else {
+            v = s < SP ? ws[(size_t)row0 * SP + s] : INF_F;
+        }
         st0[s] = v;
         st1[s] = INF_F;
-        if (s < SP) ws[(size_t)init_row * SP + s] = v;
     }
     if (tid < 16) { st0[SCAP + tid] = INF_F; st1[SCAP + tid] = INF_F; }
-    if (tid == 0) offs[init_row] = 0.0;
+    if (tid == 0 && s0 == 0) offs[row0] = 0.0;
 
-    // step i consumes frame f(i) = i (alpha) or L-1-i (beta) and produces the row stored for
-    // frame f(i)+1 (alpha) or f(i)-1 (beta)
-    const int nsteps = L - 1;
-    const long long wstep = dir ? -(long long)SP : (long long)SP;
-    float* wp = ws + (size_t)init_row * SP + wstep;
-    const int ostep = dir ? -1 : 1;
-    double* op = offs + init_row + ostep;
+    RecCursor cur;
+    cur.wstep = dir ? -(long long)SP : (long long)SP;
+    cur.wp = ws + (size_t)row0 * SP + cur.wstep;
+    cur.ostep = dir ? -1 : 1;
+    cur.op = offs + row0 + cur.ostep;
+    cur.c = s0 == 0 ? 0.0 : offs[row0];
+    cur.pending = false;
     lds_barrier();
+    for (int i = s0; i < s1; i += 2) {
+        recurse_step<THREADS, J, KT>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
+        if (i + 1 < s1)
+            recurse_step<THREADS, J, KT>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
+    }
+}
 
-    double c = 0.0;
+// Fallback for the largest sequences: same arithmetic, edge tables re-read from memory each frame
+// instead of living in registers.
+template <int THREADS>
+__device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
+                                                        float* __restrict__ st0, float* __restrict__ st1,
+                                                        const float* __restrict__ am0, const float* __restrict__ am1,
+                                                        float* __restrict__ wmin, const int SCAP) {
+    constexpr int NW = THREADS / 64;
+    const int tid = threadIdx.x;
+    const int L = m.L, SP = m.SP, T = a.T;
+    const long long soff = state_off(m.edge_begin, b);
+    const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
+    float* ws = (dir ? a.beta : a.alpha) + (size_t)T * soff;
+    double* offs = (dir ? a.offB : a.offA) + (size_t)b * T;
+    const int K = dir ? m.Kout : m.Kin;
+    int s0, s1;
+    step_range(L, dir, a.nch, a.launch, &s0, &s1);
+    const int init_state = dir ? m.end_local : m.start_local;
+    const int row0 = dir ? L - 1 - s0 : s0;
+    for (int s = tid; s < SCAP; s += THREADS) {
+        float v;
+        if (s0 == 0) {
+            v = s == init_state ? 0.f : INF_F;
+            if (s < SP) ws[(size_t)row0 * SP + s] = v;
+        } else {
+            v = s < SP ? ws[(size_t)row0 * SP + s] : INF_F;
+        }
+        st0[s] = v;
+        st1[s] = INF_F;
+    }
+    if (tid < 16) { st0[SCAP + tid] = INF_F; st1[SCAP + tid] = INF_F; }
+    if (tid == 0 && s0 == 0) offs[row0] = 0.0;
+    const long long wstep = dir ? -(long long)SP : (long long)SP;
+    float* wp = ws + (size_t)row0 * SP + wstep;
+    const int ostep = dir ? -1 : 1;
+    double* op = offs + row0 + ostep;
+    double c = s0 == 0 ? 0.0 : offs[row0];
     bool pending = false;
     float* stc = st0; float* stn = st1;
     const float* amc = am0; const float* amn = am1;
-    for (int i = 0; i < nsteps; i++) {
+    lds_barrier();
+    for (int i = s0; i < s1; i++) {
         float pend = 0.f;
         if (pending) {
             float mn = wmin[0];
 #pragma unroll
             for (int w = 1; w < NW; w++) mn = fminf(mn, wmin[w]);
             pend = mn == INF_F ? 0.f : mn;
+            c += (double)pend;
         }
-        c += (double)pend;
         float rmin = INF_F;
-#pragma unroll
-        for (int j = 0; j < J; j++) {
-            const int s = tid + j * THREADS;
-            float v[KT];
+        for (int s = tid; s < SP; s += THREADS) {
+            float v[KMAX];
             float mn = INF_F;
 #pragma unroll
-            for (int k = 0; k < KT; k++) {
-                v[k] = (stc[eo[j][k]] - pend) + (ew[j][k] + amc[es[j][k]]);
-                mn = fminf(mn, v[k]);
+            for (int k = 0; k < KMAX; k++) {
+                v[k] = INF_F;
+                if (k < K) {
+                    const uint2 r = ell[(size_t)k * SP + s];
+                    const unsigned other = r.x & 0xFFFFu;
+                    if (other != NO_STATE) v[k] = stc[other] + (__uint_as_float(r.y) + amc[r.x >> 16]);
+                    mn = fminf(mn, v[k]);
+                }
             }
             float sum = 0.f;
 #pragma unroll
-            for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f((mn - v[k]) * 1.44269504088896341f);
-            // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
-            const float r = mn == INF_F ? INF_F : mn - 0.693147180559945309f * __builtin_amdgcn_logf(sum);
+            for (int k = 0; k < KMAX; k++) sum += __builtin_amdgcn_exp2f(mn - v[k]);
+            const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
             stn[s] = r;
-            if (s < SP) wp[s] = r;
+            wp[s] = r;
             rmin = fminf(rmin, r);
         }
         if (tid == 0) *op = c;
         wp += wstep; op += ostep;
         pending = (i % RENORM) == RENORM - 1;
         if (pending) {
-            rmin = wave_min(rmin);
-            if ((tid & 63) == 0) wmin[tid >> 6] = rmin;
+            rmin = wave_min_dpp(rmin);
+            if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
         }
         lds_barrier();
         float* t_ = stc; stc = stn; stn = t_;
@@ -493,7 +706,7 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
 
 // Loader wave: keeps the compact emission rows of the next P frames in flight (registers)
 // and drops the row of frame f(i+1) into the idle LDS buffer during step i.  It issues no
-// global stores, so its loads retire in order and the wait counts stay exact.
+// global stores, so its wait counts stay exact.
 template <int THREADS, int JL, int P>
 __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
                                              float* __restrict__ am0, float* __restrict__ am1) {
@@ -502,29 +715,30 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     const int L = m.L, DP = m.DP, T = a.T;
     const long long goff = slot_off(m.edge_begin, b);
     const float* G = a.gtab + (size_t)T * goff;
-    const int nsteps = L - 1;
+    int s0, s1;
+    step_range(L, dir, a.nch, a.launch, &s0, &s1);
     const int nchunk = DP >> 2;                       // DP is a multiple of 16
     int cc[JL];                                       // my float4 chunks of a row (clamped)
 #pragma unroll
     for (int jl = 0; jl < JL; jl++) cc[jl] = min(lane + jl * 64, nchunk - 1);
-    // row consumed by step i (clamped to the steps that exist)
+    // row consumed by step i (clamped to the steps of this launch)
     auto rowp = [&](int i) -> const f4* {
-        const int ic = min(i, nsteps - 1);
+        const int ic = min(i, s1 - 1);
         return (const f4*)(G + (size_t)(dir ? L - 1 - ic : ic) * DP);
     };
     f4 g[P][JL];
-    if (nsteps > 0) {
+    if (s1 > s0) {
 #pragma unroll
-        for (int jl = 0; jl < JL; jl++) ((f4*)am0)[lane + jl * 64] = rowp(0)[cc[jl]];
+        for (int jl = 0; jl < JL; jl++) ((f4*)am0)[lane + jl * 64] = rowp(s0)[cc[jl]];
 #pragma unroll
         for (int p = 0; p < P; p++)
 #pragma unroll
-            for (int jl = 0; jl < JL; jl++) g[p][jl] = rowp(1 + p)[cc[jl]];
+            for (int jl = 0; jl < JL; jl++) g[p][jl] = rowp(s0 + 1 + p)[cc[jl]];
     }
     lds_barrier();
     f4* amn = (f4*)am1; f4* amc = (f4*)am0;
-    int i0 = 0;
-    for (; i0 + P <= nsteps; i0 += P) {
+    int i0 = s0;
+    for (; i0 + P <= s1; i0 += P) {
 #pragma unroll
         for (int q = 0; q < P; q++) {
             const f4* nxt = rowp(i0 + q + 1 + P);
@@ -539,7 +753,7 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     }
 #pragma unroll
     for (int q = 0; q < P; q++) {
-        if (i0 + q < nsteps) {
+        if (i0 + q < s1) {
 #pragma unroll
             for (int jl = 0; jl < JL; jl++) amn[lane + jl * 64] = g[q][jl];
             lds_barrier();
@@ -548,29 +762,38 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     }
 }
 
-// THREADS compute threads plus one loader wave per workgroup.
-template <int THREADS, int J, int JL, int P, int CLS>
-__global__ __launch_bounds__(THREADS + 64) void fbw_recurse(RecArgs a) {
-    constexpr int SCAP = THREADS * J, DCAP = 256 * JL, NW = THREADS / 64;
-    __shared__ float st[2][SCAP + 16];
-    __shared__ __attribute__((aligned(16))) float amr[2][DCAP];
+// REC_THREADS compute threads plus one loader wave per workgroup; grid = 2B.
+__global__ __launch_bounds__(REC_THREADS + 64) void fbw_recurse(RecArgs a) {
+    constexpr int T_ = REC_THREADS, NW = T_ / 64;
+    __shared__ float st[2][S_MAX + 16];
+    __shared__ __attribute__((aligned(16))) float amr[2][D_MAX];
     __shared__ float wmin[NW];
 
     const int b = blockIdx.x >> 1, dir = blockIdx.x & 1;
     const SeqMeta m = a.meta[b];
-    if (rec_class(m) != CLS) return;
-    if (threadIdx.x >= THREADS) {
-        recurse_load<THREADS, JL, P>(a, m, b, dir, amr[0], amr[1]);
-        return;
-    }
+    const int cls = rec_class(m);
+    if (cls <= 0) return;
+    const bool loader = threadIdx.x >= T_;
     const int K = dir ? m.Kout : m.Kin;
-    // the loop body is specialised on the number of edge slots per state so that all LDS
-    // reads of a frame are issued back to back; unused slots point at the +inf cell
-    if (K <= 2) recurse_compute<THREADS, J, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-    else if (K <= 3) recurse_compute<THREADS, J, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-    else if (K <= 4) recurse_compute<THREADS, J, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-    else if (K <= 6) recurse_compute<THREADS, J, 6>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-    else recurse_compute<THREADS, J, KMAX>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+    // The loop body is specialised on the number of states per thread and of edge slots per state,
+    // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
+    if (cls == 1) {
+        if (loader) recurse_load<T_, 2, 8>(a, m, b, dir, amr[0], amr[1]);
+        else if (K <= 2) recurse_compute<T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 3) recurse_compute<T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 4) recurse_compute<T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 6) recurse_compute<T_, 1, 6>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else recurse_compute<T_, 1, KMAX>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+    } else if (cls == 2) {
+        if (loader) recurse_load<T_, 8, 2>(a, m, b, dir, amr[0], amr[1]);
+        else if (K <= 2) recurse_compute<T_, 4, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 3) recurse_compute<T_, 4, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 4) recurse_compute<T_, 4, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else recurse_compute_generic<T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, 4 * T_);
+    } else {
+        if (loader) recurse_load<T_, 16, 1>(a, m, b, dir, amr[0], amr[1]);
+        else recurse_compute_generic<T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, S_MAX);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -583,50 +806,103 @@ struct CombArgs {
     const SeqMeta* meta; const uint4* crec; const int* cbegin; const int* demis;
     const float* alpha; const float* beta; const float* gtab; const double* offA; const double* offB;
     float* out; float* sum_output;
-    int xs_cap;
+    int nch, k0, k1;     // this launch covers chunks k0 (blockIdx.z == 0) and k1 (blockIdx.z == 1)
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef float float4a __attribute__((ext_vector_type(4)));
 
-__device__ inline void stream_const_row(float* dst, int F, float v) {
-    const float4u c = {v, v, v, v};
-    const int n4 = F >> 2;
-    for (int i = threadIdx.x; i < n4; i += COMB_THREADS) __builtin_nontemporal_store(c, (float4u*)(dst + 4 * i));
-    const int tail = F & 3;
-    if ((int)threadIdx.x < tail) dst[4 * n4 + threadIdx.x] = v;
+// Row streaming.  Rows start at arbitrary 4-byte offsets (F need not be a multiple of 32), so the
+// row is addressed from the 128-byte line boundary below its start: chunk c covers floats
+// [4c, 4c+4) counted from that boundary, every wave store starts on a line boundary, and only the
+// chunks cut by the row's ends fall back to scalar stores.  The line-aligned chunks go out as
+// non-temporal stores: the tensor is written once and never read here, and keeping it out of the
+// caches measured faster for the whole call (I6_NT=0 switches to plain stores).
+#ifndef I6_NT
+#define I6_NT 1
+#endif
+#if I6_NT
+#define I6_ROW_STORE(v, p) __builtin_nontemporal_store(v, p)
+#else
+#define I6_ROW_STORE(v, p) (*(p) = (v))
+#endif
+__device__ __forceinline__ int row_misalign(const float* row) { return (int)(((uintptr_t)row >> 2) & 31); }
+
+__device__ inline void stream_const_row(float* row, int F, float v) {
+    const int a = row_misalign(row);
+    float* base = row - a;
+    const float4a c = {v, v, v, v};
+    const int ch_lo = (a + 3) >> 2, ch_hi = (a + F) >> 2;      // chunks that lie completely inside the row
+    for (int ch = threadIdx.x; ch < ch_hi; ch += COMB_THREADS)
+        if (ch >= ch_lo) I6_ROW_STORE(c, (float4a*)(base + 4 * ch));
+    if (threadIdx.x < 8) {                                      // the floats of the two cut chunks
+        const int i = threadIdx.x < 4 ? 4 * (ch_lo - 1) + threadIdx.x : 4 * ch_hi + threadIdx.x - 4;
+        if (i >= a && i < a + F && (i < 4 * ch_lo || i >= 4 * ch_hi)) base[i] = v;
+    }
 }
 
-template <int CLS>
+// image[a + f] holds column f of the row; a = row_misalign(row)
+__device__ inline void stream_image_row(float* row, int F, const float4a* lds4, const float* image) {
+    const int a = row_misalign(row);
+    float* base = row - a;
+    const int ch_lo = (a + 3) >> 2, ch_hi = (a + F) >> 2;
+    constexpr int U = 4;                                        // LDS reads in flight per thread
+    for (int c0 = threadIdx.x; c0 < ch_hi; c0 += U * COMB_THREADS) {
+        float4a v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int ch = c0 + u * COMB_THREADS;
+            if (ch < ch_hi) v[u] = lds4[ch];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int ch = c0 + u * COMB_THREADS;
+            if (ch >= ch_lo && ch < ch_hi) I6_ROW_STORE(v[u], (float4a*)(base + 4 * ch));
+        }
+    }
+    if (threadIdx.x < 8) {
+        const int i = threadIdx.x < 4 ? 4 * (ch_lo - 1) + threadIdx.x : 4 * ch_hi + threadIdx.x - 4;
+        if (i >= a && i < a + F && (i < 4 * ch_lo || i >= 4 * ch_hi)) base[i] = image[i];
+    }
+}
+
+__device__ __forceinline__ float block_min256(float v, float* red) {
+    v = wave_min_dpp(v);
+    if ((threadIdx.x & 63) == 63) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fminf(fminf(red[0], red[1]), fminf(red[2], red[3]));
+}
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+    v = wave_sum_dpp(v);
+    if ((threadIdx.x & 63) == 63) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
 __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
-    constexpr int NW = COMB_THREADS / 64;
+    static_assert(COMB_THREADS == 256, "block reductions assume 4 waves");
 
-    const int b = blockIdx.y, t0 = blockIdx.x * TC, tid = threadIdx.x;
+    // sequence index fastest: workgroups that run together write neighbouring rows
+    const int b = blockIdx.x, tid = threadIdx.x;
     const SeqMeta m = a.meta[b];
-    if (comb_class(m) != CLS) return;
+    if (seq_error(m) || m.n_edges == 0 || m.L == 0) return;      // fbw_padfill writes those rows
     const int T = a.T, B = a.B, F = a.F;
-    const int t1 = min(T, t0 + TC);
+    const int kc = blockIdx.z ? a.k1 : a.k0;
+    const int c1 = chunk_lo(m.L, kc + 1, a.nch);
+    const int t0 = chunk_lo(m.L, kc, a.nch) + blockIdx.y * TC;
+    if (t0 >= c1) return;
+    const int tv = min(c1, t0 + TC);    // frames [t0, tv) of this strip, all of them carry mass
     const bool prob = a.out_mode == I6FBW_OUT_PROB;
     const float hole = prob ? 0.f : INF_F;
-    const int err = seq_error(m);
-    const int L = (err || m.n_edges == 0) ? 0 : m.L;
-
-    if (t0 >= L) {   // nothing but padding (or an unusable sequence) in this strip
-        const float v = err ? __builtin_nanf("") : hole;
-        for (int t = t0; t < t1; t++) {
-            stream_const_row(a.out + ((size_t)t * B + b) * F, F, v);
-            if (tid == 0) a.sum_output[(size_t)t * B + b] = err ? __builtin_nanf("") : 0.f;
-        }
-        return;
-    }
 
     float* image = (float*)lds4;
-    const int F4 = (F + 3) >> 2;
+    const int F4 = (F + 32 + 3) >> 2;     // the image is shifted by the row's offset within its 128-byte line
     float* xs = image + 4 * F4;
     for (int i = tid; i < F4; i += COMB_THREADS) lds4[i] = (float4a){hole, hole, hole, hole};
+    int a_prev = -1;                      // image shift of the previous frame
 
     const int nE = m.n_edges, D = m.D, SP = m.SP, DP = m.DP;
     const long long soff = state_off(m.edge_begin, b), goff = slot_off(m.edge_begin, b);
@@ -635,91 +911,166 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     const int* de = a.demis + goff;
     const double* offA = a.offA + (size_t)b * T;
     const double* offB = a.offB + (size_t)b * T;
+    const float* abase = a.alpha + (size_t)T * soff;
+    const float* bbase = a.beta + (size_t)T * soff;
+    const float* gbase = a.gtab + (size_t)T * goff;
 
-    for (int t = t0; t < t1; t++) {
-        float* orow = a.out + ((size_t)t * B + b) * F;
-        if (t >= L) {
-            stream_const_row(orow, F, hole);
-            if (tid == 0) a.sum_output[(size_t)t * B + b] = 0.f;
-            continue;
-        }
-        const float* arow = a.alpha + (size_t)T * soff + (size_t)t * SP;
-        const float* brow = a.beta + (size_t)T * soff + (size_t)t * SP;
-        const float* grow = a.gtab + (size_t)T * goff + (size_t)t * DP;
-
-        // edge scores x = alpha_t[from] + w + am + beta_{t+1}[to]   (fbw_op.cu:93-100)
-        float lmin = INF_F;
-        for (int i = tid; i < nE; i += COMB_THREADS) {
-            const uint4 r = crec[i];
-            const float x = arow[r.x & 0xFFFFu] + __uint_as_float(r.y) + grow[r.z] + brow[r.x >> 16];
-            xs[i] = x;
-            lmin = fminf(lmin, x);
-        }
-        lmin = wave_min(lmin);
-        if ((tid & 63) == 0) redmin[tid >> 6] = lmin;
-        __syncthreads();
-        float mn = redmin[0];
-#pragma unroll
-        for (int w = 1; w < NW; w++) mn = fminf(mn, redmin[w]);
+    // writes the image positions of one frame from the per-slot sums, then streams the row out
+    auto finish_row = [&](int t, float mn, float tot, const float* sd, const int* em, int nslot_regs, double offs) {
         const bool dead = mn == INF_F;
-        for (int i = tid; i < nE; i += COMB_THREADS) xs[i] = dead ? 0.f : __expf(mn - xs[i]);
-        __syncthreads();
-
-        // per-emission sums in fixed (input) order, then the frame normaliser  (fbw_op.cu:115-134)
-        float sd[COMB_JD];
-        float lsum = 0.f;
-#pragma unroll
-        for (int jd = 0; jd < COMB_JD; jd++) {
-            const int d = tid + jd * COMB_THREADS;
-            float s = 0.f;
-            if (d < D) {
-                const int e0 = cb[d], e1 = cb[d + 1];
-                for (int i = e0; i < e1; i++) s += xs[i];
-            }
-            sd[jd] = s;
-            lsum += s;
-        }
-        lsum = wave_sum(lsum);
-        if ((tid & 63) == 0) redsum[tid >> 6] = lsum;
-        __syncthreads();
-        float tot = redsum[0];
-#pragma unroll
-        for (int w = 1; w < NW; w++) tot += redsum[w];
-        const float logtot = __logf(tot);
+        const float logtot = __builtin_amdgcn_logf(tot);
         if (tid == 0)
-            a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)((double)(mn + -logtot) + offA[t] + offB[t]);
+            a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)(((double)(mn - logtot) + offs) * (double)LN2);
         const float inv = dead ? 0.f : 1.f / tot;
-#pragma unroll
-        for (int jd = 0; jd < COMB_JD; jd++) {
-            const int d = tid + jd * COMB_THREADS;
+        float* orow = a.out + ((size_t)t * B + b) * F;
+        const int sh = row_misalign(orow);
+        if (a_prev >= 0 && a_prev != sh) {
+            for (int js = 0; js < nslot_regs; js++)
+                if (tid + js * COMB_THREADS < D) image[a_prev + em[js]] = hole;
+            __syncthreads();
+        }
+        a_prev = sh;
+        for (int js = 0; js < nslot_regs; js++) {
+            const int d = tid + js * COMB_THREADS;
             if (d < D) {
                 float v;
-                if (prob) v = sd[jd] * inv;
-                else v = (dead || sd[jd] == 0.f) ? INF_F : logtot - __logf(sd[jd]);
-                image[de[d]] = v;
+                if (prob) v = sd[js] * inv;
+                else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+                image[sh + em[js]] = v;
             }
         }
         __syncthreads();
-        const int n4 = F >> 2;
-        for (int i = tid; i < n4; i += COMB_THREADS) __builtin_nontemporal_store((float4u)lds4[i], (float4u*)(orow + 4 * i));
-        const int tail = F & 3;
-        if (tid < tail) orow[4 * n4 + tid] = image[4 * n4 + tid];
+        stream_image_row(orow, F, lds4, image);
+    };
+
+    if (nE <= COMB_XS && D <= 2 * COMB_THREADS) {
+        // fast path: this thread's edges and slots stay in registers for the whole strip, and
+        // the operands of the next frame are fetched while the current one is processed
+        constexpr int JE = COMB_XS / COMB_THREADS, JS = 2;
+        unsigned efr[JE], eto[JE], esl[JE];
+        float ew[JE];
+#pragma unroll
+        for (int j = 0; j < JE; j++) {
+            const int i = tid + j * COMB_THREADS;
+            uint4 r = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+            if (i < nE) r = crec[i];
+            efr[j] = r.x & 0xFFFFu; eto[j] = r.x >> 16; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
+        }
+        int c0[JS], c1[JS], em[JS];
+#pragma unroll
+        for (int js = 0; js < JS; js++) {
+            const int d = tid + js * COMB_THREADS;
+            c0[js] = c1[js] = em[js] = 0;
+            if (d < D) { c0[js] = cb[d]; c1[js] = cb[d + 1]; em[js] = de[d]; }
+        }
+        float va[JE], vb[JE], vg[JE];
+        double voff = 0.0;
+        auto fetch = [&](int t) {
+            const float* arow = abase + (size_t)t * SP;
+            const float* brow = bbase + (size_t)t * SP;
+            const float* grow = gbase + (size_t)t * DP;
+#pragma unroll
+            for (int j = 0; j < JE; j++) { va[j] = arow[efr[j]]; vb[j] = brow[eto[j]]; vg[j] = grow[esl[j]]; }
+            if (tid == 0) voff = offA[t] + offB[t];
+        };
+        fetch(t0);
+        for (int t = t0; t < tv; t++) {
+            // edge scores x = alpha_t[from] + w + am + beta_{t+1}[to]   (fbw_op.cu:93-100)
+            float x[JE];
+            float lmin = INF_F;
+#pragma unroll
+            for (int j = 0; j < JE; j++) { x[j] = (va[j] + ew[j]) + (vg[j] + vb[j]); lmin = fminf(lmin, x[j]); }
+            const double offs = voff;
+            if (t + 1 < tv) fetch(t + 1);
+            const float mn = block_min256(lmin, redmin);
+#pragma unroll
+            for (int j = 0; j < JE; j++) xs[tid + j * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
+            __syncthreads();
+            // per-emission sums in fixed (input) order, then the frame normaliser (fbw_op.cu:115-134)
+            float sd[JS];
+            float lsum = 0.f;
+#pragma unroll
+            for (int js = 0; js < JS; js++) {
+                float s = 0.f;
+                for (int i = c0[js]; i < c1[js]; i++) s += xs[i];
+                sd[js] = s;
+                lsum += s;
+            }
+            const float tot = block_sum256(lsum, redsum);
+            finish_row(t, mn, tot, sd, em, JS, offs);
+        }
+    } else {
+        // general path: edge records re-read per frame, edges staged through LDS in passes of
+        // COMB_XS, per-slot sums accumulated across the passes
+        for (int t = t0; t < tv; t++) {
+            const float* arow = abase + (size_t)t * SP;
+            const float* brow = bbase + (size_t)t * SP;
+            const float* grow = gbase + (size_t)t * DP;
+            auto score = [&](int i) {
+                const uint4 r = crec[i];
+                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + (grow[r.z] + brow[r.x >> 16]);
+            };
+            float lmin = INF_F;
+            for (int i = tid; i < nE; i += COMB_THREADS) lmin = fminf(lmin, score(i));
+            const float mn = block_min256(lmin, redmin);
+            float sd[COMB_JD];
+            int em[COMB_JD];
+#pragma unroll
+            for (int jd = 0; jd < COMB_JD; jd++) { sd[jd] = 0.f; em[jd] = 0; }
+            for (int p0 = 0; p0 < nE; p0 += COMB_XS) {
+                const int p1 = min(nE, p0 + COMB_XS);
+                __syncthreads();
+                for (int i = p0 + tid; i < p1; i += COMB_THREADS)
+                    xs[i - p0] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - score(i));
+                __syncthreads();
+#pragma unroll
+                for (int jd = 0; jd < COMB_JD; jd++) {
+                    const int d = tid + jd * COMB_THREADS;
+                    if (d < D) {
+                        const int e0 = max(cb[d], p0), e1 = min(cb[d + 1], p1);
+                        float s = sd[jd];
+                        for (int i = e0; i < e1; i++) s += xs[i - p0];
+                        sd[jd] = s;
+                    }
+                }
+            }
+            float lsum = 0.f;
+#pragma unroll
+            for (int jd = 0; jd < COMB_JD; jd++) {
+                const int d = tid + jd * COMB_THREADS;
+                if (d < D) em[jd] = de[d];
+                lsum += sd[jd];
+            }
+            const float tot = block_sum256(lsum, redsum);
+            finish_row(t, mn, tot, sd, em, COMB_JD, offA[t] + offB[t]);
+        }
+    }
+}
+
+// Rows that carry no probability mass: frames t >= seq_len, and every frame of a sequence without
+// edges, with seq_len outside [1, T] (out = hole, sum_output = 0: fbw_op.cu:120-128,366-369) or
+// with a reported problem (NaN).  These rows depend on nothing but the meta records.
+__global__ __launch_bounds__(COMB_THREADS) void fbw_padfill(CombArgs a) {
+    const int b = blockIdx.x, t0 = blockIdx.y * TC;
+    const SeqMeta m = a.meta[b];
+    const int err = seq_error(m);
+    const int L = (err || m.n_edges == 0) ? 0 : m.L;
+    const int t1 = min(a.T, t0 + TC);
+    const float hole = a.out_mode == I6FBW_OUT_PROB ? 0.f : INF_F;
+    const float v = err ? __builtin_nanf("") : hole;
+    for (int t = max(t0, L); t < t1; t++) {
+        stream_const_row(a.out + ((size_t)t * a.B + b) * a.F, a.F, v);
+        if (threadIdx.x == 0) a.sum_output[(size_t)t * a.B + b] = err ? __builtin_nanf("") : 0.f;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-thread_local hipError_t g_last_hip_error = hipSuccess;
+constexpr int MAX_CHUNKS = 32;
+constexpr int MAX_DEVICES = 64;
 
-struct Profile {
-    bool on = false;
-    int calls = 0;
-    static constexpr int MAXREC = 256;
-    hipEvent_t ev[MAXREC][I6FBW_N_STAGES + 1];
-    bool created = false;
-};
-Profile g_prof;
+thread_local hipError_t g_last_hip_error = hipSuccess;
 
 #define HIP_TRY(expr)                                              \
     do {                                                           \
@@ -727,7 +1078,78 @@ Profile g_prof;
         if (e_ != hipSuccess) { g_last_hip_error = e_; return I6FBW_ERR_LAUNCH; } \
     } while (0)
 
-size_t comb_lds_bytes(int F, int xs_cap) { return (size_t)(((F + 3) >> 2) * 16) + (size_t)xs_cap * 4; }
+// Library-owned streams and events of one device.  A call forks from the caller's stream after
+// the edge preparation, runs gather / recursion / dense write on three streams that hand time
+// chunks to each other through events, and joins the caller's stream again at the end.
+struct Pipeline {
+    bool ready = false;
+    hipStream_t sG = nullptr, sR = nullptr, sC = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    hipEvent_t evG[MAX_CHUNKS], evR[MAX_CHUNKS];
+};
+Pipeline g_pipe[MAX_DEVICES];
+std::mutex g_mutex;
+
+int pipeline_init(Pipeline& p) {
+    if (p.ready) return I6FBW_OK;
+    // default priority on purpose
+    HIP_TRY(hipStreamCreateWithFlags(&p.sG, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&p.sC, hipStreamNonBlocking));
+    HIP_TRY(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
+    HIP_TRY(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
+    for (int i = 0; i < MAX_CHUNKS; i++) {
+        HIP_TRY(hipEventCreateWithFlags(&p.evG[i], hipEventDisableTiming));
+        HIP_TRY(hipEventCreateWithFlags(&p.evR[i], hipEventDisableTiming));
+    }
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    p.ready = true;
+    return I6FBW_OK;
+}
+
+// Stage timing: event pairs around every launch of a stage, on the stream it runs on.
+struct Profile {
+    bool on = false;
+    static constexpr int MAXPAIR = 8192;
+    int n_pairs = 0, n_calls = 0;
+    hipEvent_t a[MAXPAIR], b[MAXPAIR];
+    int stage[MAXPAIR];
+    int n_created = 0;
+};
+Profile g_prof;
+
+struct StageTimer {
+    int idx = -1;
+    hipStream_t stream;
+    StageTimer(int stage, hipStream_t st) : stream(st) {
+        if (!g_prof.on || g_prof.n_pairs >= Profile::MAXPAIR) return;
+        if (g_prof.n_pairs >= g_prof.n_created) {
+            if (hipEventCreate(&g_prof.a[g_prof.n_created]) != hipSuccess) return;
+            if (hipEventCreate(&g_prof.b[g_prof.n_created]) != hipSuccess) return;
+            g_prof.n_created++;
+        }
+        idx = g_prof.n_pairs++;
+        g_prof.stage[idx] = stage;
+        (void)hipEventRecord(g_prof.a[idx], stream);
+    }
+    ~StageTimer() {
+        if (idx >= 0) (void)hipEventRecord(g_prof.b[idx], stream);
+    }
+};
+
+size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
+
+int env_chunks() {
+    static const int n = [] {
+        const char* e = getenv("I6FBW_CHUNKS");
+        int v = e ? atoi(e) : 1;
+        if (v < 1) v = 1;
+        if (v > MAX_CHUNKS) v = MAX_CHUNKS;
+        if (v > 1 && (v & 1)) v++;      // chunks pair up from both ends
+        return v;
+    }();
+    return n;
+}
 
 }  // namespace
 
@@ -748,83 +1170,113 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     if (E > 0 && (!edges || !weights)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
-    if (B > 65535) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
     const Layout l = make_layout(T, B, E);
     if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
-    const int xs_small = 1024, xs_large = EB_MAX;
-    const bool need_large = E > 1024;
-    if (F > F_BITMAP_MAX || comb_lds_bytes(F, need_large ? xs_large : xs_small) > 160 * 1024 - 256) return I6FBW_ERR_F_TOO_LARGE;
+    if (F > F_BITMAP_MAX || comb_lds_bytes(F) > 160 * 1024 - 256) return I6FBW_ERR_F_TOO_LARGE;
 
-    hipStream_t stream = (hipStream_t)stream_;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    Pipeline& P = g_pipe[dev];
+    { int rc = pipeline_init(P); if (rc != I6FBW_OK) return rc; }
+
+    hipStream_t s = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     SeqMeta* meta = (SeqMeta*)(ws + l.meta);
-
-    hipEvent_t* ev = nullptr;
-    if (g_prof.on) {
-        if (!g_prof.created) {
-            for (int i = 0; i < Profile::MAXREC; i++)
-                for (int s = 0; s <= I6FBW_N_STAGES; s++) HIP_TRY(hipEventCreate(&g_prof.ev[i][s]));
-            g_prof.created = true;
-        }
-        if (g_prof.calls < Profile::MAXREC) ev = g_prof.ev[g_prof.calls++];
-    }
-    if (ev) HIP_TRY(hipEventRecord(ev[0], stream));
+    // One chunk (the default) keeps everything on the caller's stream.  I6FBW_CHUNKS=n (even) cuts
+    // the time axis into n chunks and overlaps gather, recursion and dense write across the three
+    // library streams; on this runtime the event hand-offs between streams cost more than the
+    // overlap gains, so it is off unless asked for.
+    const int nch = T >= 256 ? env_chunks() : 1;
+    const bool piped = nch > 1;
+    hipStream_t sG = piped ? P.sG : s, sR = piped ? P.sR : s, sC = piped ? P.sC : s;
+    if (g_prof.on) g_prof.n_calls++;
 
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
     pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states;
-    pa.meta = meta; pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
+    pa.meta = meta; pa.sortflag = (int*)(ws + l.sortflag); pa.eidx = (int*)(ws + l.eidx);
+    pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis);
-    hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, stream, pa);
-    HIP_TRY(hipGetLastError());
-    if (ev) HIP_TRY(hipEventRecord(ev[1], stream));
-
-    GatherArgs ga;
-    ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
-    ga.meta = meta; ga.demis = pa.demis; ga.gtab = (float*)(ws + l.gtab);
-    hipLaunchKernelGGL(fbw_gather, dim3((T + TG - 1) / TG, B), dim3(256), 0, stream, ga);
-    HIP_TRY(hipGetLastError());
-    if (ev) HIP_TRY(hipEventRecord(ev[2], stream));
-
-    RecArgs ra;
-    ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
-    ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
-    ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB);
-    hipLaunchKernelGGL((fbw_recurse<512, 1, 2, 8, 1>), dim3(2 * B), dim3(512 + 64), 0, stream, ra);
-    HIP_TRY(hipGetLastError());
-    // a sequence can only be in a larger class if the batch has that many states or emissions
-    if (n_states > 512 || (E > 512 && F > 512)) {
-        hipLaunchKernelGGL((fbw_recurse<512, 4, 8, 4, 2>), dim3(2 * B), dim3(512 + 64), 0, stream, ra);
+    {
+        StageTimer tm(0, s);
+        if (E > 0) {
+            hipLaunchKernelGGL(fbw_scan_sorted, dim3((E + SCAN_BLOCK - 1) / SCAN_BLOCK), dim3(256), 0, s,
+                               edges + 3 * edge_row_stride, E, pa.sortflag);
+            HIP_TRY(hipGetLastError());
+        }
+        hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
         HIP_TRY(hipGetLastError());
     }
-    if (n_states > 2048 || (E > 2048 && F > 2048)) {
-        hipLaunchKernelGGL((fbw_recurse<512, 8, 16, 2, 3>), dim3(2 * B), dim3(512 + 64), 0, stream, ra);
-        HIP_TRY(hipGetLastError());
+    if (piped) {
+        HIP_TRY(hipEventRecord(P.fork, s));
+        HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
+        HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
+        HIP_TRY(hipStreamWaitEvent(sC, P.fork, 0));
     }
-    if (ev) HIP_TRY(hipEventRecord(ev[3], stream));
 
     CombArgs ca;
     ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
-    ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
-    ca.out = out; ca.sum_output = sum_output;
-    static bool attr_set = false;
-    if (!attr_set) {
-        HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        attr_set = true;
-    }
-    const dim3 cgrid((T + TC - 1) / TC, B);
-    ca.xs_cap = xs_small;
-    hipLaunchKernelGGL(fbw_combine<1>, cgrid, dim3(COMB_THREADS), comb_lds_bytes(F, xs_small), stream, ca);
-    HIP_TRY(hipGetLastError());
-    if (need_large) {
-        ca.xs_cap = xs_large;
-        hipLaunchKernelGGL(fbw_combine<2>, cgrid, dim3(COMB_THREADS), comb_lds_bytes(F, xs_large), stream, ca);
+    ca.alpha = (float*)(ws + l.alpha); ca.beta = (float*)(ws + l.beta); ca.gtab = (float*)(ws + l.gtab);
+    ca.offA = (double*)(ws + l.offA); ca.offB = (double*)(ws + l.offB);
+    ca.out = out; ca.sum_output = sum_output; ca.nch = nch; ca.k0 = 0; ca.k1 = 0;
+    {   // rows without probability mass depend on the meta records only
+        StageTimer tm(4, sC);
+        hipLaunchKernelGGL(fbw_padfill, dim3(B, (T + TC - 1) / TC), dim3(COMB_THREADS), 0, sC, ca);
         HIP_TRY(hipGetLastError());
     }
-    if (ev) HIP_TRY(hipEventRecord(ev[4], stream));
+
+    GatherArgs ga;
+    ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
+    ga.meta = meta; ga.demis = pa.demis; ga.gtab = (float*)(ws + l.gtab); ga.nch = nch;
+    RecArgs ra;
+    ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
+    ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
+    ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.nch = nch;
+    const int chunk_frames = (T + nch - 1) / nch + 1;       // longest chunk of any sequence
+    const int g_strips = (chunk_frames + TG - 1) / TG, c_strips = (chunk_frames + TC - 1) / TC;
+    const int n_pairs = piped ? nch / 2 : 1, nz = piped ? 2 : 1;
+
+    // gather: chunk pairs from the outside in, in the order the recursions consume them
+    for (int i = 0; i < n_pairs; i++) {
+        ga.k0 = i; ga.k1 = nch - 1 - i;
+        {
+            StageTimer tm(1, sG);
+            hipLaunchKernelGGL(fbw_gather, dim3(g_strips, B, nz), dim3(256), 0, sG, ga);
+            HIP_TRY(hipGetLastError());
+        }
+        if (piped) HIP_TRY(hipEventRecord(P.evG[i], sG));
+    }
+    // recursion: launch j moves alpha over chunk j and beta over chunk nch-1-j
+    for (int j = 0; j < nch; j++) {
+        if (piped && j < n_pairs) HIP_TRY(hipStreamWaitEvent(sR, P.evG[j], 0));
+        ra.launch = j;
+        {
+            StageTimer tm(2, sR);
+            hipLaunchKernelGGL(fbw_recurse, dim3(2 * B), dim3(REC_THREADS + 64), 0, sR, ra);
+            HIP_TRY(hipGetLastError());
+        }
+        if (piped) HIP_TRY(hipEventRecord(P.evR[j], sR));
+    }
+    // combine: chunks k and nch-1-k have both directions once launch max(k, nch-1-k) is done
+    for (int j = piped ? nch / 2 : 0; j < nch; j++) {
+        if (piped) HIP_TRY(hipStreamWaitEvent(sC, P.evR[j], 0));
+        ca.k0 = nch - 1 - j; ca.k1 = j;
+        {
+            StageTimer tm(3, sC);
+            hipLaunchKernelGGL(fbw_combine, dim3(B, c_strips, nz), dim3(COMB_THREADS), comb_lds_bytes(F), sC, ca);
+            HIP_TRY(hipGetLastError());
+        }
+    }
+    if (piped) {
+        // sC has waited for the last recursion launch, which has waited for every gather
+        HIP_TRY(hipEventRecord(P.join, sC));
+        HIP_TRY(hipStreamWaitEvent(s, P.join, 0));
+    }
     return I6FBW_OK;
 }
 
@@ -864,24 +1316,26 @@ const char* i6fbw_strerror(int code) {
 const char* i6fbw_last_hip_error(void) { return g_last_hip_error == hipSuccess ? "" : hipGetErrorString(g_last_hip_error); }
 
 void i6fbw_profile_enable(int on) {
+    std::lock_guard<std::mutex> lock(g_mutex);
     g_prof.on = on != 0;
-    g_prof.calls = 0;
+    g_prof.n_pairs = 0;
+    g_prof.n_calls = 0;
 }
 
 int i6fbw_profile_read(float* stage_ms) {
-    const int n = g_prof.calls;
-    for (int s = 0; s < I6FBW_N_STAGES; s++) stage_ms[s] = 0.f;
-    if (n == 0) return 0;
-    for (int i = 0; i < n; i++) {
-        if (hipEventSynchronize(g_prof.ev[i][I6FBW_N_STAGES]) != hipSuccess) return 0;
-        for (int s = 0; s < I6FBW_N_STAGES; s++) {
-            float ms = 0.f;
-            hipEventElapsedTime(&ms, g_prof.ev[i][s], g_prof.ev[i][s + 1]);
-            stage_ms[s] += ms / n;
-        }
+    std::lock_guard<std::mutex> lock(g_mutex);
+    for (int st = 0; st < I6FBW_N_STAGES; st++) stage_ms[st] = 0.f;
+    const int calls = g_prof.n_calls;
+    if (calls == 0) return 0;
+    for (int i = 0; i < g_prof.n_pairs; i++) {
+        float ms = 0.f;
+        if (hipEventSynchronize(g_prof.b[i]) != hipSuccess) continue;
+        if (hipEventElapsedTime(&ms, g_prof.a[i], g_prof.b[i]) != hipSuccess) continue;
+        stage_ms[g_prof.stage[i]] += ms / calls;
     }
-    g_prof.calls = 0;
-    return n;
+    g_prof.n_pairs = 0;
+    g_prof.n_calls = 0;
+    return calls;
 }
 
 }  // extern "C"

@@ -64,7 +64,10 @@ int i6fbw_workspace_size(int T, int B, int F, int E, int n_states, size_t* bytes
  *   sum_output  float [T,B] contiguous: total -log likelihood of sequence b in every frame
  *               t < seq_lens[b], 0 elsewhere                         (fbw_op.cu:104-135,232)
  *   workspace   device buffer of at least i6fbw_workspace_size bytes, 256-byte aligned
- *   stream      hipStream_t to enqueue on (NULL = default stream); the call is asynchronous
+ *   stream      hipStream_t to enqueue on (NULL = default stream); the call is asynchronous.
+ *               Inside, the work forks onto library-owned streams (created on first use, default
+ *               priority) and joins `stream` again before the call returns, so everything
+ *               enqueued on `stream` afterwards sees the finished outputs.
  *
  * Returns I6FBW_OK or a negative host-side status.  Problems only the device can
  * see (index out of range, an automaton beyond the supported size) are recorded in
@@ -95,15 +98,17 @@ const char* i6fbw_strerror(int code);
 const char* i6fbw_last_hip_error(void);
 
 /*
- * Average device time in milliseconds of each pipeline stage over all i6fbw_run
- * calls since the last reset, measured with HIP events on the stream the kernels
- * ran on.  Stage timing is off by default; i6fbw_profile_enable(1) turns it on
- * (it adds event records between stages), i6fbw_profile_enable(0) turns it off
- * and clears the sums.  stage_ms has room for I6FBW_N_STAGES entries:
- * 0 edge preparation, 1 emission gather, 2 alpha/beta recursion, 3 combine + dense write.
- * Waits for the recorded events.  Returns the number of calls averaged over.
+ * Average device time per call, in milliseconds, of each stage over all i6fbw_run calls since
+ * profiling was switched on, measured with HIP event pairs around every launch of the stage on
+ * the stream that launch runs on (the stages of one call overlap in time, so the entries do not
+ * add up to the call's duration).  Off by default; i6fbw_profile_enable(1) turns it on and clears
+ * the sums, i6fbw_profile_enable(0) turns it off.  stage_ms has room for I6FBW_N_STAGES entries:
+ * 0 edge preparation, 1 emission gather, 2 alpha/beta recursion, 3 combine + dense write of the
+ * frames that carry probability mass, 4 fill of the remaining rows.  Keeps at most 8192 launches.
+ * i6fbw_profile_read waits for the recorded events, returns the number of calls averaged over
+ * and clears the sums.
  */
-#define I6FBW_N_STAGES 4
+#define I6FBW_N_STAGES 5
 void i6fbw_profile_enable(int on);
 int i6fbw_profile_read(float* stage_ms);
 
