@@ -17,6 +17,7 @@ STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
+           "i6fbw_set_overlap",
            "i6fbw_profile_enable", "i6fbw_profile_read")
 
 _lib = None
@@ -40,6 +41,8 @@ def load():
         lib.i6fbw_strerror.argtypes = [c.c_int]
         lib.i6fbw_strerror.restype = c.c_char_p
         lib.i6fbw_last_hip_error.restype = c.c_char_p
+        lib.i6fbw_set_overlap.argtypes = [c.c_int]
+        lib.i6fbw_set_overlap.restype = None
         lib.i6fbw_profile_enable.argtypes = [c.c_int]
         lib.i6fbw_profile_enable.restype = None
         lib.i6fbw_profile_read.argtypes = [c.POINTER(c.c_float)]
@@ -79,6 +82,11 @@ def read_status(ws_ptr, B, stream=0):
     if rc != 0:
         raise FbwError(rc)
     return int(code.value), int(seq.value)
+
+
+def set_overlap(mode: int) -> None:
+    """-1: by problem size, 0: single stream, 1: overlapped stages."""
+    load().i6fbw_set_overlap(int(mode))
 
 
 def profile_enable(on: bool) -> None:

@@ -49,6 +49,10 @@ constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of t
 constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup (plus one loader wave)
 constexpr unsigned NO_STATE = 0xFFFFu;
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
+constexpr int SYNC_HDR = 16;          // ints before the progress counters in the hand-off area:
+                                      // [0] abort flag, [1] recursion workgroups placed so far
+constexpr int PUBLISH = 32;           // recursion steps between progress publications
+constexpr int SPIN_LIMIT = 1 << 20;   // polls before a waiting wave gives up
 // Scores are kept in units of log 2 inside the workspace (exp2/log2 are single instructions).
 constexpr float LOG2E = 1.44269504088896341f;
 constexpr float LN2 = 0.693147180559945309f;
@@ -75,7 +79,7 @@ __host__ __device__ inline long long state_off(long long edge_begin, int b) { re
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 
 struct Layout {
-    size_t meta, sortflag, eidx, ellA, ellB, crec, cbegin, demis, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sync, sortflag, eidx, ellA, ellB, crec, cbegin, demis, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
 };
 
@@ -87,6 +91,7 @@ Layout make_layout(long long T, long long B, long long E) {
     l.gg_total = round16(E) + 32 * B + 16;
     size_t o = 0;
     l.meta = o;     o = align256(o + sizeof(SeqMeta) * B);
+    l.sync = o;     o = align256(o + sizeof(int) * (SYNC_HDR + 2 * B + B * ((T + TG - 1) / TG)));
     l.sortflag = o; o = align256(o + sizeof(int) * (E / SCAN_BLOCK + 2));
     l.eidx = o;     o = align256(o + sizeof(int) * (E + 1));
     l.ellA = o;     o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
@@ -117,8 +122,36 @@ __device__ inline int rec_class(const SeqMeta& m) {
     return 3;
 }
 
-// The frames [0, L) of a sequence are cut into nch chunks; chunk k covers [chunk_lo(k), chunk_lo(k+1)).
-__device__ __forceinline__ int chunk_lo(int L, int k, int nch) { return (int)((long long)k * L / nch); }
+// Hand-off between kernels that run at the same time (gather -> recursion -> combine).  The
+// L2 caches of the eight XCDs are not coherent with each other inside a kernel, so everything
+// that crosses kernels goes through agent-scope accesses (sc1: written through / read from the
+// memory side), and a flag or counter is published only after the data stores have completed.
+// Every wait is bounded: after SPIN_LIMIT polls the waiter sets the abort flag and goes on, and
+// the call reports I6FBW_ERR_TIMEOUT.
+__device__ __forceinline__ void store_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_agent(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void store_agent(double* p, double v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ int load_agent(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ double load_agent(const double* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ unsigned long long load_agent(const unsigned long long* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool SYNC, typename T> __device__ __forceinline__ void store_x(T* p, T v) { if (SYNC) store_agent(p, v); else *p = v; }
+template <bool SYNC, typename T> __device__ __forceinline__ T load_x(const T* p) { return SYNC ? load_agent(p) : *p; }
+// waits until this wave's global stores have been acknowledged
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// polls *p until it is >= want; false if it gave up (or somebody else already had to)
+__device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort_flag) {
+    for (int n = 0; n < SPIN_LIMIT; n++) {
+        if (load_agent(p) >= want) return true;
+        if ((n & 255) == 255 && load_agent(abort_flag)) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+    atomicOr(abort_flag, 1);
+    return false;
+}
 
 // wave-wide minimum in lane 63 (DPP row operations, no LDS traffic)
 __device__ __forceinline__ float wave_min_dpp(float v) {
@@ -160,7 +193,7 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
-    SeqMeta* meta; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis;
+    SeqMeta* meta; int* sync; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis;
 };
 
 // sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never decrease
@@ -331,6 +364,14 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
+    if (role == 2) {
+        // hand-off area of this sequence: progress counters and gather flags start at zero
+        const int nstrip = (a.T + TG - 1) / TG;
+        if (b == 0 && tid < SYNC_HDR) a.sync[tid] = 0;
+        if (tid < 2) a.sync[SYNC_HDR + 2 * b + tid] = 0;
+        int* gf = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * nstrip;
+        for (int i = tid; i < nstrip; i += 1024) gf[i] = 0;
+    }
     if (role == 2 && tid == 0) {
         SeqMeta* m = a.meta + b;
         m->edge_begin = edge_begin; m->n_edges = n_edges; m->state_min = (int)smin;
@@ -433,28 +474,32 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// stage 2: gather  gtab[b][t][slot] = log2(e) * am[t, b, demis[b][slot]]  for t < L_b
+// stage 2: gather  gtab[b][t][slot] = log2(e) * am[t, b, demis[b][slot]]  for t < L_b.
+// Strips of TG frames are handed out from both ends of a sequence towards its middle, the order in
+// which the two recursions consume them.  With SYNC the rows are written through and a flag per
+// strip tells the recursion (running at the same time) that the strip is complete.
 // ---------------------------------------------------------------------------------------------
 struct GatherArgs {
     const float* am; long long st_t, st_b;
     int T, B;
     const SeqMeta* meta; const int* demis; float* gtab;
-    int nch, k0, k1;     // this launch covers chunks k0 (blockIdx.z == 0) and k1 (blockIdx.z == 1)
+    int* sync;
 };
 
+template <bool SYNC>
 __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
-    const int b = blockIdx.y;
+    const int b = blockIdx.x, y = blockIdx.y;
     const SeqMeta m = a.meta[b];
     if (rec_class(m) <= 0) return;
-    const int k = blockIdx.z ? a.k1 : a.k0;
-    const int c0 = chunk_lo(m.L, k, a.nch), c1 = chunk_lo(m.L, k + 1, a.nch);
-    const int t0 = c0 + blockIdx.x * TG;
-    if (t0 >= c1) return;
+    const int n = (m.L + TG - 1) / TG;
+    if (y >= n) return;
+    const int j = (y & 1) ? n - 1 - (y >> 1) : (y >> 1);
+    const int t0 = j * TG;
     const long long goff = slot_off(m.edge_begin, b);
     const int* de = a.demis + goff;
     float* g = a.gtab + (size_t)a.T * goff;
     const float* am = a.am + (long long)b * a.st_b;
-    const int nt = min(TG, c1 - t0);
+    const int nt = min(TG, m.L - t0);
     for (int idx = threadIdx.x; idx < m.DP; idx += 256) {
         const int e = de[idx];
         float v[TG];
@@ -463,7 +508,12 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
             if (tt < nt) v[tt] = am[(long long)(t0 + tt) * a.st_t + e];
 #pragma unroll
         for (int tt = 0; tt < TG; tt++)
-            if (tt < nt) g[(size_t)(t0 + tt) * m.DP + idx] = v[tt] * LOG2E;
+            if (tt < nt) store_x<SYNC>(&g[(size_t)(t0 + tt) * m.DP + idx], v[tt] * LOG2E);
+    }
+    if (SYNC) {
+        wait_stores();
+        __syncthreads();
+        if (threadIdx.x == 0) store_agent(&a.sync[SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG) + j], 1);
     }
 }
 
@@ -471,43 +521,43 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
 // stage 3: recursion.  Workgroup 2b walks alpha of sequence b forward, workgroup 2b+1 walks beta
 // backward.  Rows stored for frame t: alpha_t (state vector before frame t is consumed) and
 // beta_{t+1} (after it), in units of log 2, each relative to an offset kept in double precision.
+// With SYNC the loader wave waits for the gather flags, the rows are written through, and the
+// number of finished rows is published every PUBLISH steps for the combine kernel.
 // ---------------------------------------------------------------------------------------------
 struct RecArgs {
     int T, B;
     const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab;
     float* alpha; float* beta; double* offA; double* offB;
-    int nch, launch;     // launch j advances alpha over chunk j and beta over chunk nch-1-j
+    int* sync;
 };
 
-// Steps [*s0, *s1) of direction dir that belong to launch `launch`.  Step i consumes frame i (alpha)
-// or L-1-i (beta); there are L-1 steps in all.
-__device__ __forceinline__ void step_range(int L, int dir, int nch, int launch, int* s0, int* s1) {
-    if (!dir) {
-        *s0 = chunk_lo(L, launch, nch);
-        *s1 = min(chunk_lo(L, launch + 1, nch), L - 1);
-    } else {
-        const int k = nch - 1 - launch;
-        *s0 = L - chunk_lo(L, k + 1, nch);
-        *s1 = L - max(chunk_lo(L, k, nch), 1);
-    }
-    if (*s1 < *s0) *s1 = *s0;
-}
-
 // Barrier for LDS traffic only: waits for this wave's LDS operations and not for its global
-// memory traffic (the compute waves' row stores, the loader wave's prefetches).
+// memory traffic (the compute waves' row stores, the loader wave's prefetches).  The memory
+// clobber is what tells the compiler that other waves change the LDS buffers in between, so the
+// pointers to those buffers must not be declared restrict.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 struct RecCursor {
     float* wp; long long wstep;      // workspace row written by the next step
     double* op; int ostep;           // its offset
     double c; bool pending;          // running offset, renormalisation requested by the last step
+    int* progress; int nsteps;       // rows finished so far (SYNC), number of steps
 };
+
+// end of a step: optional publication of the progress counter, and the per-frame barrier
+template <bool SYNC>
+__device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
+    const bool pub = SYNC && (((i + 1) % PUBLISH) == 0 || i + 1 == cur.nsteps);
+    if (pub) wait_stores();          // every compute wave: its rows up to this step are out
+    lds_barrier();
+    if (pub && threadIdx.x == 0) store_agent(cur.progress, i + 2);
+}
 
 // One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
 // LDS, log-sum-exp (base 2) in a fixed order, result to the other LDS buffer and the workspace.
-template <int THREADS, int J, int KT>
-__device__ __forceinline__ void recurse_step(const int i, const int SP, const char* __restrict__ stc, float* __restrict__ stn,
-                                             const char* __restrict__ amc, float* __restrict__ wmin,
+template <bool SYNC, int THREADS, int J, int KT>
+__device__ __forceinline__ void recurse_step(const int i, const int SP, const char* stc, float* stn,
+                                             const char* amc, float* wmin,
                                              const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
                                              const float (&ew)[J][KT], RecCursor& cur) {
     constexpr int NW = THREADS / 64;
@@ -537,31 +587,63 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
         const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
         stn[s] = r;
-        if (s < SP) cur.wp[s] = r;
+        if (s < SP) store_x<SYNC>(cur.wp + s, r);
         rmin = fminf(rmin, r);
     }
-    if (tid == 0) *cur.op = cur.c;
+    if (tid == 0) store_x<SYNC>(cur.op, cur.c);
     cur.wp += cur.wstep; cur.op += cur.ostep;
     cur.pending = (i % RENORM) == RENORM - 1;
     if (cur.pending) {
         rmin = wave_min_dpp(rmin);
         if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
     }
-    lds_barrier();
+    step_end<SYNC>(i, cur);
 }
 
-template <int THREADS, int J, int KT>
-__device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                                float* __restrict__ st0, float* __restrict__ st1,
-                                                const float* __restrict__ am0, const float* __restrict__ am1,
-                                                float* __restrict__ wmin) {
-    constexpr int SCAP = THREADS * J;
+// common prologue of the compute waves: initial state vector, row 0 of the workspace, cursor
+template <bool SYNC, int THREADS>
+__device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int SCAP,
+                                             float* st0, float* st1, RecCursor& cur) {
     const int tid = threadIdx.x;
     const int L = m.L, SP = m.SP, T = a.T;
     const long long soff = state_off(m.edge_begin, b);
-    const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
     float* ws = (dir ? a.beta : a.alpha) + (size_t)T * soff;
     double* offs = (dir ? a.offB : a.offA) + (size_t)b * T;
+    const int init_state = dir ? m.end_local : m.start_local;
+    const int row0 = dir ? L - 1 : 0;
+    for (int s = tid; s < SCAP; s += THREADS) {
+        const float v = s == init_state ? 0.f : INF_F;
+        st0[s] = v;
+        st1[s] = INF_F;
+        if (s < SP) store_x<SYNC>(&ws[(size_t)row0 * SP + s], v);
+    }
+    if (tid < 16) { st0[SCAP + tid] = INF_F; st1[SCAP + tid] = INF_F; }
+    if (tid == 0) store_x<SYNC>(&offs[row0], 0.0);
+    // step i consumes frame f(i) = i (alpha) or L-1-i (beta) and produces the row stored for
+    // frame f(i)+1 (alpha) or f(i)-1 (beta); L-1 steps in all
+    cur.wstep = dir ? -(long long)SP : (long long)SP;
+    cur.wp = ws + (size_t)row0 * SP + cur.wstep;
+    cur.ostep = dir ? -1 : 1;
+    cur.op = offs + row0 + cur.ostep;
+    cur.c = 0.0;
+    cur.pending = false;
+    cur.progress = a.sync + SYNC_HDR + 2 * b + dir;
+    cur.nsteps = L - 1;
+    if (SYNC) wait_stores();
+    lds_barrier();
+    if (SYNC && tid == 0) store_agent(cur.progress, 1);      // the initial row is out
+}
+
+template <bool SYNC, int THREADS, int J, int KT>
+__device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
+                                                float* st0, float* st1,
+                                                const float* am0, const float* am1,
+                                                float* wmin) {
+    constexpr int SCAP = THREADS * J;
+    const int tid = threadIdx.x;
+    const int SP = m.SP;
+    const long long soff = state_off(m.edge_begin, b);
+    const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
     const int K = dir ? m.Kout : m.Kin;
 
     // edges of my states -> registers, as LDS byte offsets of the other state / the emission slot
@@ -581,93 +663,40 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
             ew[j][k] = __uint_as_float(r.y);
         }
     }
-
-    // state before the first step of this launch: the initial vector, or the row an earlier
-    // launch stored (values relative to the offset stored beside it)
-    int s0, s1;
-    step_range(L, dir, a.nch, a.launch, &s0, &s1);
-    const int init_state = dir ? m.end_local : m.start_local;
-    const int row0 = dir ? L - 1 - s0 : s0;
-#pragma unroll
-    for (int j = 0; j < J; j++) {
-        const int s = tid + j * THREADS;
-        float v;
-        if (s0 == 0) {
-            v = s == init_state ? 0.f : INF_F;
-            if (s < SP) ws[(size_t)row0 * SP + s] = v;
-        } else {
-            v = s < SP ? ws[(size_t)row0 * SP + s] : INF_F;
-        }
-        st0[s] = v;
-        st1[s] = INF_F;
-    }
-    if (tid < 16) { st0[SCAP + tid] = INF_F; st1[SCAP + tid] = INF_F; }
-    if (tid == 0 && s0 == 0) offs[row0] = 0.0;
-
     RecCursor cur;
-    cur.wstep = dir ? -(long long)SP : (long long)SP;
-    cur.wp = ws + (size_t)row0 * SP + cur.wstep;
-    cur.ostep = dir ? -1 : 1;
-    cur.op = offs + row0 + cur.ostep;
-    cur.c = s0 == 0 ? 0.0 : offs[row0];
-    cur.pending = false;
-    lds_barrier();
-    for (int i = s0; i < s1; i += 2) {
-        recurse_step<THREADS, J, KT>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
-        if (i + 1 < s1)
-            recurse_step<THREADS, J, KT>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
+    recurse_init<SYNC, THREADS>(a, m, b, dir, SCAP, st0, st1, cur);
+    for (int i = 0; i < cur.nsteps; i += 2) {
+        recurse_step<SYNC, THREADS, J, KT>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
+        if (i + 1 < cur.nsteps)
+            recurse_step<SYNC, THREADS, J, KT>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
     }
 }
 
 // Fallback for the largest sequences: same arithmetic, edge tables re-read from memory each frame
 // instead of living in registers.
-template <int THREADS>
+template <bool SYNC, int THREADS>
 __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                                        float* __restrict__ st0, float* __restrict__ st1,
-                                                        const float* __restrict__ am0, const float* __restrict__ am1,
-                                                        float* __restrict__ wmin, const int SCAP) {
+                                                        float* st0, float* st1,
+                                                        const float* am0, const float* am1,
+                                                        float* wmin, const int SCAP) {
     constexpr int NW = THREADS / 64;
     const int tid = threadIdx.x;
-    const int L = m.L, SP = m.SP, T = a.T;
+    const int SP = m.SP;
     const long long soff = state_off(m.edge_begin, b);
     const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
-    float* ws = (dir ? a.beta : a.alpha) + (size_t)T * soff;
-    double* offs = (dir ? a.offB : a.offA) + (size_t)b * T;
     const int K = dir ? m.Kout : m.Kin;
-    int s0, s1;
-    step_range(L, dir, a.nch, a.launch, &s0, &s1);
-    const int init_state = dir ? m.end_local : m.start_local;
-    const int row0 = dir ? L - 1 - s0 : s0;
-    for (int s = tid; s < SCAP; s += THREADS) {
-        float v;
-        if (s0 == 0) {
-            v = s == init_state ? 0.f : INF_F;
-            if (s < SP) ws[(size_t)row0 * SP + s] = v;
-        } else {
-            v = s < SP ? ws[(size_t)row0 * SP + s] : INF_F;
-        }
-        st0[s] = v;
-        st1[s] = INF_F;
-    }
-    if (tid < 16) { st0[SCAP + tid] = INF_F; st1[SCAP + tid] = INF_F; }
-    if (tid == 0 && s0 == 0) offs[row0] = 0.0;
-    const long long wstep = dir ? -(long long)SP : (long long)SP;
-    float* wp = ws + (size_t)row0 * SP + wstep;
-    const int ostep = dir ? -1 : 1;
-    double* op = offs + row0 + ostep;
-    double c = s0 == 0 ? 0.0 : offs[row0];
-    bool pending = false;
+    RecCursor cur;
+    recurse_init<SYNC, THREADS>(a, m, b, dir, SCAP, st0, st1, cur);
     float* stc = st0; float* stn = st1;
     const float* amc = am0; const float* amn = am1;
-    lds_barrier();
-    for (int i = s0; i < s1; i++) {
+    for (int i = 0; i < cur.nsteps; i++) {
         float pend = 0.f;
-        if (pending) {
+        if (cur.pending) {
             float mn = wmin[0];
 #pragma unroll
             for (int w = 1; w < NW; w++) mn = fminf(mn, wmin[w]);
             pend = mn == INF_F ? 0.f : mn;
-            c += (double)pend;
+            cur.c += (double)pend;
         }
         float rmin = INF_F;
         for (int s = tid; s < SP; s += THREADS) {
@@ -688,87 +717,104 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
             for (int k = 0; k < KMAX; k++) sum += __builtin_amdgcn_exp2f(mn - v[k]);
             const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
             stn[s] = r;
-            wp[s] = r;
+            store_x<SYNC>(cur.wp + s, r);
             rmin = fminf(rmin, r);
         }
-        if (tid == 0) *op = c;
-        wp += wstep; op += ostep;
-        pending = (i % RENORM) == RENORM - 1;
-        if (pending) {
+        if (tid == 0) store_x<SYNC>(cur.op, cur.c);
+        cur.wp += cur.wstep; cur.op += cur.ostep;
+        cur.pending = (i % RENORM) == RENORM - 1;
+        if (cur.pending) {
             rmin = wave_min_dpp(rmin);
             if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
         }
-        lds_barrier();
+        step_end<SYNC>(i, cur);
         float* t_ = stc; stc = stn; stn = t_;
         const float* u_ = amc; amc = amn; amn = u_;
     }
 }
 
-// Loader wave: keeps the compact emission rows of the next P frames in flight (registers)
-// and drops the row of frame f(i+1) into the idle LDS buffer during step i.  It issues no
-// global stores, so its wait counts stay exact.
-template <int THREADS, int JL, int P>
+// Loader wave: keeps the compact emission rows of the next P frames in flight (registers, 8-byte
+// pieces) and drops the row of frame f(i+1) into the idle LDS buffer during step i.  It issues
+// no global stores, so its wait counts stay exact.  With SYNC it first makes sure the gather
+// kernel has finished the strip a row belongs to.
+template <bool SYNC, int THREADS, int JL, int P>
 __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                             float* __restrict__ am0, float* __restrict__ am1) {
-    typedef float f4 __attribute__((ext_vector_type(4)));
+                                             float* am0, float* am1) {
+    typedef unsigned long long u64;
     const int lane = threadIdx.x - THREADS;
     const int L = m.L, DP = m.DP, T = a.T;
     const long long goff = slot_off(m.edge_begin, b);
     const float* G = a.gtab + (size_t)T * goff;
-    int s0, s1;
-    step_range(L, dir, a.nch, a.launch, &s0, &s1);
-    const int nchunk = DP >> 2;                       // DP is a multiple of 16
-    int cc[JL];                                       // my float4 chunks of a row (clamped)
-#pragma unroll
-    for (int jl = 0; jl < JL; jl++) cc[jl] = min(lane + jl * 64, nchunk - 1);
-    // row consumed by step i (clamped to the steps of this launch)
-    auto rowp = [&](int i) -> const f4* {
-        const int ic = min(i, s1 - 1);
-        return (const f4*)(G + (size_t)(dir ? L - 1 - ic : ic) * DP);
+    const int nsteps = L - 1;
+    const int npiece = DP >> 1;                       // DP is a multiple of 16
+    // my pieces of a row: lane + jl*64, clamped to the row
+    auto cc = [&](int jl) { return min(lane + jl * 64, npiece - 1); };
+    int* abort_flag = a.sync;
+    const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((T + TG - 1) / TG);
+    int strip_ok = -1;
+    // row consumed by step i (clamped to the steps that exist); waits for its strip first
+    auto rowp = [&](int i) -> const u64* {
+        const int ic = min(i, nsteps - 1);
+        const int f = dir ? L - 1 - ic : ic;
+        if (SYNC && f / TG != strip_ok) {
+            spin_until_ge(gflag + f / TG, 1, abort_flag);
+            strip_ok = f / TG;
+        }
+        return (const u64*)(G + (size_t)f * DP);
     };
-    f4 g[P][JL];
-    if (s1 > s0) {
+    u64 g[P][JL];
+    if (nsteps > 0) {
+        const u64* r0 = rowp(0);
 #pragma unroll
-        for (int jl = 0; jl < JL; jl++) ((f4*)am0)[lane + jl * 64] = rowp(s0)[cc[jl]];
+        for (int jl = 0; jl < JL; jl++) ((u64*)am0)[lane + jl * 64] = load_x<SYNC>(r0 + cc(jl));
 #pragma unroll
-        for (int p = 0; p < P; p++)
+        for (int p = 0; p < P; p++) {
+            const u64* rp = rowp(1 + p);
 #pragma unroll
-            for (int jl = 0; jl < JL; jl++) g[p][jl] = rowp(s0 + 1 + p)[cc[jl]];
+            for (int jl = 0; jl < JL; jl++) g[p][jl] = load_x<SYNC>(rp + cc(jl));
+        }
     }
-    lds_barrier();
-    f4* amn = (f4*)am1; f4* amc = (f4*)am0;
-    int i0 = s0;
-    for (; i0 + P <= s1; i0 += P) {
+    lds_barrier();      // pairs with the barrier at the end of recurse_init
+    u64* amn = (u64*)am1; u64* amc = (u64*)am0;
+    int i0 = 0;
+    for (; i0 + P <= nsteps; i0 += P) {
 #pragma unroll
         for (int q = 0; q < P; q++) {
-            const f4* nxt = rowp(i0 + q + 1 + P);
+            const u64* nxt = rowp(i0 + q + 1 + P);
 #pragma unroll
             for (int jl = 0; jl < JL; jl++) {
                 amn[lane + jl * 64] = g[q][jl];
-                g[q][jl] = nxt[cc[jl]];
+                g[q][jl] = load_x<SYNC>(nxt + cc(jl));
             }
             lds_barrier();
-            f4* t_ = amc; amc = amn; amn = t_;
+            u64* t_ = amc; amc = amn; amn = t_;
         }
     }
 #pragma unroll
     for (int q = 0; q < P; q++) {
-        if (i0 + q < s1) {
+        if (i0 + q < nsteps) {
 #pragma unroll
             for (int jl = 0; jl < JL; jl++) amn[lane + jl * 64] = g[q][jl];
             lds_barrier();
-            f4* t_ = amc; amc = amn; amn = t_;
+            u64* t_ = amc; amc = amn; amn = t_;
         }
     }
 }
 
 // REC_THREADS compute threads plus one loader wave per workgroup; grid = 2B.
-__global__ __launch_bounds__(REC_THREADS + 64) void fbw_recurse(RecArgs a) {
+// DENSE caps the register use (5 waves per SIMD) so that two workgroups fit on a compute unit;
+// the host picks it when the batch has more workgroups than the device has compute units.  The
+// rarely used large-automaton paths pay for the cap with spills, which is why small batches run
+// the uncapped instance.
+template <bool SYNC, bool DENSE>
+__global__ __launch_bounds__(REC_THREADS + 64, DENSE ? 5 : 1) void fbw_recurse(RecArgs a) {
     constexpr int T_ = REC_THREADS, NW = T_ / 64;
     __shared__ float st[2][S_MAX + 16];
     __shared__ __attribute__((aligned(16))) float amr[2][D_MAX];
     __shared__ float wmin[NW];
 
+    // every workgroup reports that it has been placed (see fbw_gate)
+    if (SYNC && threadIdx.x == 0) atomicAdd(&a.sync[1], 1);
     const int b = blockIdx.x >> 1, dir = blockIdx.x & 1;
     const SeqMeta m = a.meta[b];
     const int cls = rec_class(m);
@@ -778,21 +824,21 @@ __global__ __launch_bounds__(REC_THREADS + 64) void fbw_recurse(RecArgs a) {
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     if (cls == 1) {
-        if (loader) recurse_load<T_, 2, 8>(a, m, b, dir, amr[0], amr[1]);
-        else if (K <= 2) recurse_compute<T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 3) recurse_compute<T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 4) recurse_compute<T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 6) recurse_compute<T_, 1, 6>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else recurse_compute<T_, 1, KMAX>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        if (loader) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
+        else if (K <= 2) recurse_compute<SYNC, T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 3) recurse_compute<SYNC, T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 4) recurse_compute<SYNC, T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 6) recurse_compute<SYNC, T_, 1, 6>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else recurse_compute<SYNC, T_, 1, KMAX>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
     } else if (cls == 2) {
-        if (loader) recurse_load<T_, 8, 2>(a, m, b, dir, amr[0], amr[1]);
-        else if (K <= 2) recurse_compute<T_, 4, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 3) recurse_compute<T_, 4, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 4) recurse_compute<T_, 4, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else recurse_compute_generic<T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, 4 * T_);
+        if (loader) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1]);
+        else if (K <= 2) recurse_compute<SYNC, T_, 4, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 3) recurse_compute<SYNC, T_, 4, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else if (K <= 4) recurse_compute<SYNC, T_, 4, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
+        else recurse_compute_generic<SYNC, T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, 4 * T_);
     } else {
-        if (loader) recurse_load<T_, 16, 1>(a, m, b, dir, amr[0], amr[1]);
-        else recurse_compute_generic<T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, S_MAX);
+        if (loader) recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
+        else recurse_compute_generic<SYNC, T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, S_MAX);
     }
 }
 
@@ -806,7 +852,7 @@ struct CombArgs {
     const SeqMeta* meta; const uint4* crec; const int* cbegin; const int* demis;
     const float* alpha; const float* beta; const float* gtab; const double* offA; const double* offB;
     float* out; float* sum_output;
-    int nch, k0, k1;     // this launch covers chunks k0 (blockIdx.z == 0) and k1 (blockIdx.z == 1)
+    int* sync;
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -879,6 +925,7 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+template <bool SYNC>
 __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
     __shared__ float redmin[COMB_THREADS / 64];
@@ -890,11 +937,25 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     const SeqMeta m = a.meta[b];
     if (seq_error(m) || m.n_edges == 0 || m.L == 0) return;      // fbw_padfill writes those rows
     const int T = a.T, B = a.B, F = a.F;
-    const int kc = blockIdx.z ? a.k1 : a.k0;
-    const int c1 = chunk_lo(m.L, kc + 1, a.nch);
-    const int t0 = chunk_lo(m.L, kc, a.nch) + blockIdx.y * TC;
-    if (t0 >= c1) return;
-    const int tv = min(c1, t0 + TC);    // frames [t0, tv) of this strip, all of them carry mass
+    // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
+    // forward and the backward recursion meet, so those rows are complete first
+    const int n = (m.L + TC - 1) / TC, y = blockIdx.y;
+    if (y >= n) return;
+    const int strip = (y & 1) ? n / 2 - 1 - (y >> 1) : n / 2 + (y >> 1);
+    const int t0 = strip * TC;
+    const int tv = min(m.L, t0 + TC);    // frames [t0, tv) of this strip, all of them carry mass
+    if (SYNC) {
+        // alpha rows [0, count_a) and beta rows [L - count_b, L) have been written through
+        __shared__ int s_ok;
+        if (tid == 0) {
+            const int* prog = a.sync + SYNC_HDR + 2 * b;
+            bool ok = spin_until_ge(prog, tv, a.sync);
+            ok = ok && spin_until_ge(prog + 1, m.L - t0, a.sync);
+            s_ok = ok;
+        }
+        __syncthreads();
+        if (!s_ok) return;       // timed out: reported through the abort flag
+    }
     const bool prob = a.out_mode == I6FBW_OUT_PROB;
     const float hole = prob ? 0.f : INF_F;
 
@@ -970,8 +1031,10 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             const float* brow = bbase + (size_t)t * SP;
             const float* grow = gbase + (size_t)t * DP;
 #pragma unroll
-            for (int j = 0; j < JE; j++) { va[j] = arow[efr[j]]; vb[j] = brow[eto[j]]; vg[j] = grow[esl[j]]; }
-            if (tid == 0) voff = offA[t] + offB[t];
+            for (int j = 0; j < JE; j++) {
+                va[j] = load_x<SYNC>(arow + efr[j]); vb[j] = load_x<SYNC>(brow + eto[j]); vg[j] = grow[esl[j]];
+            }
+            if (tid == 0) voff = load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t);
         };
         fetch(t0);
         for (int t = t0; t < tv; t++) {
@@ -1008,7 +1071,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             const float* grow = gbase + (size_t)t * DP;
             auto score = [&](int i) {
                 const uint4 r = crec[i];
-                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + (grow[r.z] + brow[r.x >> 16]);
+                return (load_x<SYNC>(arow + (r.x & 0xFFFFu)) + __uint_as_float(r.y)) + (grow[r.z] + load_x<SYNC>(brow + (r.x >> 16)));
             };
             float lmin = INF_F;
             for (int i = tid; i < nE; i += COMB_THREADS) lmin = fminf(lmin, score(i));
@@ -1042,9 +1105,16 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
                 lsum += sd[jd];
             }
             const float tot = block_sum256(lsum, redsum);
-            finish_row(t, mn, tot, sd, em, COMB_JD, offA[t] + offB[t]);
+            finish_row(t, mn, tot, sd, em, COMB_JD, load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t));
         }
     }
+}
+
+// Holds back the combine kernel (next on the same stream) until every workgroup of the recursion
+// kernel has been placed on the machine: combine workgroups wait for recursion progress while
+// they occupy LDS and wave slots, so they must not be able to keep a recursion workgroup out.
+__global__ __launch_bounds__(64) void fbw_gate(int* sync, int need) {
+    if (threadIdx.x == 0) spin_until_ge(sync + 1, need, sync);
 }
 
 // Rows that carry no probability mass: frames t >= seq_len, and every frame of a sequence without
@@ -1078,31 +1148,32 @@ thread_local hipError_t g_last_hip_error = hipSuccess;
         if (e_ != hipSuccess) { g_last_hip_error = e_; return I6FBW_ERR_LAUNCH; } \
     } while (0)
 
-// Library-owned streams and events of one device.  A call forks from the caller's stream after
-// the edge preparation, runs gather / recursion / dense write on three streams that hand time
-// chunks to each other through events, and joins the caller's stream again at the end.
+// Library-owned streams and events of one device.  A large call forks from the caller's stream
+// after the edge preparation: the recursion stays on the caller's stream, the gather runs beside
+// it on a second stream and feeds it through flags in memory, and the dense write runs on a
+// third stream, started when the gather is done and fed by the recursion's progress counters.
 struct Pipeline {
     bool ready = false;
-    hipStream_t sG = nullptr, sR = nullptr, sC = nullptr;
-    hipEvent_t fork = nullptr, join = nullptr;
-    hipEvent_t evG[MAX_CHUNKS], evR[MAX_CHUNKS];
+    hipStream_t sG = nullptr, sC = nullptr;
+    hipEvent_t fork = nullptr, gathered = nullptr, join = nullptr;
+    int n_cu = 256;
 };
 Pipeline g_pipe[MAX_DEVICES];
 std::mutex g_mutex;
 
 int pipeline_init(Pipeline& p) {
     if (p.ready) return I6FBW_OK;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipDeviceGetAttribute(&p.n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     // default priority on purpose
     HIP_TRY(hipStreamCreateWithFlags(&p.sG, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
     HIP_TRY(hipStreamCreateWithFlags(&p.sC, hipStreamNonBlocking));
     HIP_TRY(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
+    HIP_TRY(hipEventCreateWithFlags(&p.gathered, hipEventDisableTiming));
     HIP_TRY(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
-    for (int i = 0; i < MAX_CHUNKS; i++) {
-        HIP_TRY(hipEventCreateWithFlags(&p.evG[i], hipEventDisableTiming));
-        HIP_TRY(hipEventCreateWithFlags(&p.evR[i], hipEventDisableTiming));
-    }
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     p.ready = true;
     return I6FBW_OK;
 }
@@ -1139,17 +1210,11 @@ struct StageTimer {
 
 size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
 
-int env_chunks() {
-    static const int n = [] {
-        const char* e = getenv("I6FBW_CHUNKS");
-        int v = e ? atoi(e) : 1;
-        if (v < 1) v = 1;
-        if (v > MAX_CHUNKS) v = MAX_CHUNKS;
-        if (v > 1 && (v & 1)) v++;      // chunks pair up from both ends
-        return v;
-    }();
-    return n;
-}
+// schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
+int g_overlap_mode = [] {
+    const char* e = getenv("I6FBW_OVERLAP");
+    return e ? (e[0] == '0' ? 0 : 1) : -1;
+}();
 
 }  // namespace
 
@@ -1185,20 +1250,18 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     hipStream_t s = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     SeqMeta* meta = (SeqMeta*)(ws + l.meta);
-    // One chunk (the default) keeps everything on the caller's stream.  I6FBW_CHUNKS=n (even) cuts
-    // the time axis into n chunks and overlaps gather, recursion and dense write across the three
-    // library streams; on this runtime the event hand-offs between streams cost more than the
-    // overlap gains, so it is off unless asked for.
-    const int nch = T >= 256 ? env_chunks() : 1;
-    const bool piped = nch > 1;
-    hipStream_t sG = piped ? P.sG : s, sR = piped ? P.sR : s, sC = piped ? P.sC : s;
+    int* sync = (int*)(ws + l.sync);
+    // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
+    const int forced = g_overlap_mode;
+    const bool overlap = forced >= 0 ? forced != 0 : (long long)T * B * F >= (1LL << 26);
+    hipStream_t sG = overlap ? P.sG : s, sC = overlap ? P.sC : s;
     if (g_prof.on) g_prof.n_calls++;
 
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
     pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states;
-    pa.meta = meta; pa.sortflag = (int*)(ws + l.sortflag); pa.eidx = (int*)(ws + l.eidx);
+    pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis);
     {
@@ -1211,72 +1274,59 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
         hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
         HIP_TRY(hipGetLastError());
     }
-    if (piped) {
-        HIP_TRY(hipEventRecord(P.fork, s));
-        HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
-        HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
-        HIP_TRY(hipStreamWaitEvent(sC, P.fork, 0));
-    }
-
-    CombArgs ca;
-    ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
-    ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
-    ca.alpha = (float*)(ws + l.alpha); ca.beta = (float*)(ws + l.beta); ca.gtab = (float*)(ws + l.gtab);
-    ca.offA = (double*)(ws + l.offA); ca.offB = (double*)(ws + l.offB);
-    ca.out = out; ca.sum_output = sum_output; ca.nch = nch; ca.k0 = 0; ca.k1 = 0;
-    {   // rows without probability mass depend on the meta records only
-        StageTimer tm(4, sC);
-        hipLaunchKernelGGL(fbw_padfill, dim3(B, (T + TC - 1) / TC), dim3(COMB_THREADS), 0, sC, ca);
-        HIP_TRY(hipGetLastError());
-    }
 
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
-    ga.meta = meta; ga.demis = pa.demis; ga.gtab = (float*)(ws + l.gtab); ga.nch = nch;
+    ga.meta = meta; ga.demis = pa.demis; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
     RecArgs ra;
     ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
-    ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.nch = nch;
-    const int chunk_frames = (T + nch - 1) / nch + 1;       // longest chunk of any sequence
-    const int g_strips = (chunk_frames + TG - 1) / TG, c_strips = (chunk_frames + TC - 1) / TC;
-    const int n_pairs = piped ? nch / 2 : 1, nz = piped ? 2 : 1;
+    ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.sync = sync;
+    CombArgs ca;
+    ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
+    ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
+    ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
+    ca.out = out; ca.sum_output = sum_output; ca.sync = sync;
+    const dim3 g_grid(B, (T + TG - 1) / TG), c_grid(B, (T + TC - 1) / TC);
+    const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
-    // gather: chunk pairs from the outside in, in the order the recursions consume them
-    for (int i = 0; i < n_pairs; i++) {
-        ga.k0 = i; ga.k1 = nch - 1 - i;
-        {
-            StageTimer tm(1, sG);
-            hipLaunchKernelGGL(fbw_gather, dim3(g_strips, B, nz), dim3(256), 0, sG, ga);
-            HIP_TRY(hipGetLastError());
-        }
-        if (piped) HIP_TRY(hipEventRecord(P.evG[i], sG));
+    if (!overlap) {
+        { StageTimer tm(4, s); hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, s, ca); }
+        HIP_TRY(hipGetLastError());
+        { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
+        HIP_TRY(hipGetLastError());
+        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<false, true>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra);
+          else hipLaunchKernelGGL((fbw_recurse<false, false>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra); }
+        HIP_TRY(hipGetLastError());
+        { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
+        HIP_TRY(hipGetLastError());
+        return I6FBW_OK;
     }
-    // recursion: launch j moves alpha over chunk j and beta over chunk nch-1-j
-    for (int j = 0; j < nch; j++) {
-        if (piped && j < n_pairs) HIP_TRY(hipStreamWaitEvent(sR, P.evG[j], 0));
-        ra.launch = j;
-        {
-            StageTimer tm(2, sR);
-            hipLaunchKernelGGL(fbw_recurse, dim3(2 * B), dim3(REC_THREADS + 64), 0, sR, ra);
-            HIP_TRY(hipGetLastError());
-        }
-        if (piped) HIP_TRY(hipEventRecord(P.evR[j], sR));
-    }
-    // combine: chunks k and nch-1-k have both directions once launch max(k, nch-1-k) is done
-    for (int j = piped ? nch / 2 : 0; j < nch; j++) {
-        if (piped) HIP_TRY(hipStreamWaitEvent(sC, P.evR[j], 0));
-        ca.k0 = nch - 1 - j; ca.k1 = j;
-        {
-            StageTimer tm(3, sC);
-            hipLaunchKernelGGL(fbw_combine, dim3(B, c_strips, nz), dim3(COMB_THREADS), comb_lds_bytes(F), sC, ca);
-            HIP_TRY(hipGetLastError());
-        }
-    }
-    if (piped) {
-        // sC has waited for the last recursion launch, which has waited for every gather
-        HIP_TRY(hipEventRecord(P.join, sC));
-        HIP_TRY(hipStreamWaitEvent(s, P.join, 0));
-    }
+
+    HIP_TRY(hipEventRecord(P.fork, s));
+    HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
+    HIP_TRY(hipStreamWaitEvent(sC, P.fork, 0));
+    // Enqueue order gather -> recursion -> combine: every in-kernel wait is for a kernel enqueued
+    // earlier, so the call also completes (without overlap) if the runtime maps two of the
+    // streams onto one hardware queue.
+    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(P.gathered, sG));
+    { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra);
+      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra); }
+    HIP_TRY(hipGetLastError());
+    // rows without probability mass depend on the meta records only
+    { StageTimer tm(4, sC); hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sC, ca); }
+    HIP_TRY(hipGetLastError());
+    // The dense write starts when the gather is done: by then the recursions are about to meet in
+    // the middle of the sequences, which is where the combine kernel begins.
+    HIP_TRY(hipStreamWaitEvent(sC, P.gathered, 0));
+    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sC, sync, 2 * B);
+    HIP_TRY(hipGetLastError());
+    { StageTimer tm(3, sC); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), sC, ca); }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(P.join, sC));
+    HIP_TRY(hipStreamWaitEvent(s, P.join, 0));
     return I6FBW_OK;
 }
 
@@ -1288,7 +1338,11 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
     hipError_t e = hipMemcpyAsync(host, workspace, sizeof(SeqMeta) * (size_t)B, hipMemcpyDeviceToHost, (hipStream_t)stream);
     if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) { g_last_hip_error = e; free(host); return I6FBW_ERR_LAUNCH; }
-    *code = I6FBW_OK; *seq = -1;
+    int aborted = 0;
+    // the abort flag of the hand-off area follows the meta records
+    e = hipMemcpy(&aborted, (const char*)workspace + align256(sizeof(SeqMeta) * (size_t)B), sizeof(int), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { g_last_hip_error = e; free(host); return I6FBW_ERR_LAUNCH; }
+    *code = aborted ? I6FBW_ERR_TIMEOUT : I6FBW_OK; *seq = -1;
     for (int b = 0; b < B; b++) {
         const int c = host[b].err ? host[b].err : (host[b].errA ? host[b].errA : host[b].errB);
         if (c) { *code = c; *seq = b; break; }
@@ -1309,8 +1363,14 @@ const char* i6fbw_strerror(int code) {
         case I6FBW_ERR_SEQ_DEGREE: return "a state has more than 8 incoming or outgoing edges";
         case I6FBW_ERR_SEQ_TOO_LARGE: return "a sequence has more than 4096 states or distinct emissions";
         case I6FBW_ERR_BAD_INDEX: return "sequence, emission or state index out of range";
+        case I6FBW_ERR_TIMEOUT: return "a kernel gave up waiting for another stage of the same call";
         default: return "unknown status";
     }
+}
+
+void i6fbw_set_overlap(int mode) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_overlap_mode = mode < 0 ? -1 : (mode ? 1 : 0);
 }
 
 const char* i6fbw_last_hip_error(void) { return g_last_hip_error == hipSuccess ? "" : hipGetErrorString(g_last_hip_error); }

@@ -30,7 +30,8 @@ enum {
     I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* device-side: state ids of one sequence span more than 2*edges+2 */
     I6FBW_ERR_SEQ_DEGREE = -12,           /* device-side: a state has more in- or out-edges than supported */
     I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side: states / distinct emissions of one sequence exceed LDS */
-    I6FBW_ERR_BAD_INDEX = -14             /* device-side: sequence, emission or state index out of range */
+    I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
+    I6FBW_ERR_TIMEOUT = -15               /* device-side: a stage gave up waiting for another stage of the call */
 };
 
 /* Layout of the posterior tensor written by i6fbw_run. */
@@ -90,6 +91,15 @@ int i6fbw_run(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
  * paths (fbw_op.cu:287-290, returnn_definitions.h:114-123) with a status.
  */
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq);
+
+/*
+ * Chooses how i6fbw_run schedules its stages: 0 one after the other on the caller's stream,
+ * 1 overlapped (gather, recursion and dense write run at the same time on library streams and
+ * hand frames to each other through flags in the workspace), -1 (default) overlapped for large
+ * problems only.  The environment variable I6FBW_OVERLAP=0/1 sets the initial value.  Results do
+ * not depend on the schedule.  No counterpart in the reference.
+ */
+void i6fbw_set_overlap(int mode);
 
 /* Text for a status code. */
 const char* i6fbw_strerror(int code);

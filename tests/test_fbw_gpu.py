@@ -33,6 +33,15 @@ def check_against_oracle(oracle, args, threads=1):
     return out, loss
 
 
+@pytest.fixture(params=["single_stream", "overlapped"], autouse=True)
+def schedule(request):
+    """Every parity case runs under both schedules of i6fbw_run."""
+    from i6_native_ops_amd import cabi
+    cabi.set_overlap(0 if request.param == "single_stream" else 1)
+    yield request.param
+    cabi.set_overlap(-1)
+
+
 @pytest.mark.parametrize("seq_len", [5, 4, 1, 0, 6, -3])
 def test_reference_fixture(oracle, seq_len):
     out, loss = check_against_oracle(oracle, reference_fixture(seq_len))
