@@ -46,7 +46,9 @@ constexpr int RENORM = 8;             // frames between renormalisations of the 
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
 constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of the combine kernel
-constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup (plus one loader wave)
+constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup
+constexpr int REC_LOADERS = 1;        // loader waves beside them
+constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
 constexpr unsigned NO_STATE = 0xFFFFu;
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
 constexpr int SYNC_HDR = 16;          // ints before the progress counters in the hand-off area:
@@ -544,13 +546,22 @@ struct RecCursor {
     int* progress; int nsteps;       // rows finished so far (SYNC), number of steps
 };
 
-// end of a step: optional publication of the progress counter, and the per-frame barrier
+// End of a step: the per-frame barrier and, every PUBLISH steps, the progress counter.  Stores
+// complete in issue order, so "at most PUBLISH of this wave's stores are still in flight" means
+// that every row older than PUBLISH steps has been written through (a wave issues at least one
+// store per step or none at all); publishing that older count never drains the store queue, which
+// would cost several microseconds per publication while the dense write saturates the memory.
 template <bool SYNC>
 __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
-    const bool pub = SYNC && (((i + 1) % PUBLISH) == 0 || i + 1 == cur.nsteps);
-    if (pub) wait_stores();          // every compute wave: its rows up to this step are out
+    static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
+    const bool last = i + 1 == cur.nsteps;
+    const bool pub = SYNC && (((i + 1) % PUBLISH) == 0 || last);
+    if (pub) {
+        if (last) wait_stores();
+        else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    }
     lds_barrier();
-    if (pub && threadIdx.x == 0) store_agent(cur.progress, i + 2);
+    if (pub && threadIdx.x == 0) store_agent(cur.progress, last ? i + 2 : i + 2 - PUBLISH);
 }
 
 // One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
@@ -807,7 +818,7 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
 // rarely used large-automaton paths pay for the cap with spills, which is why small batches run
 // the uncapped instance.
 template <bool SYNC, bool DENSE>
-__global__ __launch_bounds__(REC_THREADS + 64, DENSE ? 5 : 1) void fbw_recurse(RecArgs a) {
+__global__ __launch_bounds__(REC_BLOCK, DENSE ? 5 : 1) void fbw_recurse(RecArgs a) {
     constexpr int T_ = REC_THREADS, NW = T_ / 64;
     __shared__ float st[2][S_MAX + 16];
     __shared__ __attribute__((aligned(16))) float amr[2][D_MAX];
@@ -1295,8 +1306,8 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
         HIP_TRY(hipGetLastError());
         { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<false, true>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra);
-          else hipLaunchKernelGGL((fbw_recurse<false, false>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra); }
+        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<false, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
+          else hipLaunchKernelGGL((fbw_recurse<false, false>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
         { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
         HIP_TRY(hipGetLastError());
@@ -1312,8 +1323,8 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(P.gathered, sG));
-    { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra);
-      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_THREADS + 64), 0, s, ra); }
+    { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
+      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
     HIP_TRY(hipGetLastError());
     // rows without probability mass depend on the meta records only
     { StageTimer tm(4, sC); hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sC, ca); }
