@@ -81,7 +81,7 @@ __host__ __device__ inline long long state_off(long long edge_begin, int b) { re
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 
 struct Layout {
-    size_t meta, sync, sortflag, eidx, ellA, ellB, crec, cbegin, demis, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sync, sortflag, eidx, ellA, ellB, crec, cbegin, demis, tband, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
 };
 
@@ -101,6 +101,7 @@ Layout make_layout(long long T, long long B, long long E) {
     l.crec = o;     o = align256(o + sizeof(uint4) * (E + 1));
     l.cbegin = o;   o = align256(o + sizeof(int) * l.gg_total);
     l.demis = o;    o = align256(o + sizeof(int) * l.gg_total);
+    l.tband = o;    o = align256(o + sizeof(int2) * l.gg_total);
     l.offA = o;     o = align256(o + sizeof(double) * B * T);
     l.offB = o;     o = align256(o + sizeof(double) * B * T);
     l.alpha = o;    o = align256(o + sizeof(float) * l.ss_total * T);
@@ -195,7 +196,7 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
-    SeqMeta* meta; int* sync; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis;
+    SeqMeta* meta; int* sync; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
 // sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never decrease
@@ -255,6 +256,16 @@ __device__ inline int lower_bound_u32(const int32_t* a, int n, unsigned v) {
     return lo;
 }
 
+// Lower bound on the number of edges of any path from state id `from` to state id `to` when no
+// edge raises the id by more than dmax or lowers it by more than -dmin.  Exact for left-to-right
+// chains numbered along the chain; never larger than the true distance for any automaton.
+__device__ inline int min_steps(int from, int to, int dmax, int dmin) {
+    const int diff = to - from;
+    if (diff == 0) return 0;
+    if (diff > 0) return dmax > 0 ? (diff + dmax - 1) / dmax : (1 << 30);
+    return dmin < 0 ? (-diff - dmin - 1) / -dmin : (1 << 30);
+}
+
 // grid (3, B): role 0 orders the edges of sequence b by target state (alpha), role 1 by source
 // state (beta), role 2 by emission slot (combine) and writes the shared part of the meta record.
 // Edge lists grouped by sequence (the usual case) are located by binary search; any other order
@@ -264,7 +275,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     __shared__ unsigned bitmap[F_BITMAP_MAX / 32];
     __shared__ int wordpfx[F_BITMAP_MAX / 32];
     __shared__ int wsum[16];
-    __shared__ int s_lt, s_bad, s_kmax, s_sorted;
+    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin;
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -274,7 +285,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     const int32_t* e_seq = a.edges + 3 * a.edge_stride;
     const int E = a.E;
 
-    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; }
+    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; }
     __syncthreads();
     const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
     int unsorted = 0;
@@ -472,6 +483,50 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
             }
         }
         for (int d = D + tid; d < DP; d += 1024) de[d] = 0;
+
+        // Frames in which a slot can carry probability mass.  An edge u->v is dead at frame t if
+        // u cannot be reached from the start state in t edges or the end state cannot be reached
+        // from v in L-1-t edges; min_steps bounds both from below.  The gather writes +inf for
+        // (frame, slot) pairs outside [tlo, thi] instead of reading am_scores: every edge of the
+        // slot is dead there, so the result is the same, the states involved drop out of the
+        // renormalisation, and for chain-like automata about half of the gather disappears.
+        int dmax = 0, dmin = 0;
+        for (int i = tid; i < n_edges; i += 1024) {
+            const int e = edge_at(i);
+            const int df = (int)((unsigned)e_to[e] - (unsigned)e_from[e]);
+            dmax = max(dmax, df); dmin = min(dmin, df);
+        }
+        if (dmax > 0) atomicMax(&s_dmax, dmax);
+        if (dmin < 0) atomicMin(&s_dmin, dmin);
+        __syncthreads();
+        dmax = s_dmax; dmin = s_dmin;
+        const int s_loc = (int)(st_state - smin), e_loc = (int)(en_state - smin);
+        // one thread per edge; the per-slot minimum / maximum is taken with LDS atomics in the
+        // memory of the sort keys, which are not needed any more once each thread has read its own
+        constexpr int EPT = EB_MAX / 1024;
+        unsigned mykey[EPT];
+#pragma unroll
+        for (int j = 0; j < EPT; j++) mykey[j] = tid + j * 1024 < n_edges ? keys[tid + j * 1024] : ~0u;
+        __syncthreads();
+        int* s_tlo = (int*)keys;
+        int* s_thi = (int*)keys + D_MAX;
+        static_assert(2 * D_MAX <= EB_MAX, "band arrays reuse the key array");
+        for (int d = tid; d < DP; d += 1024) { s_tlo[d] = d < D ? (1 << 30) : 1; s_thi[d] = d < D ? -1 : 0; }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < EPT; j++) {
+            if (mykey[j] != ~0u) {
+                const int e = edge_at((int)(mykey[j] & POS_MASK));
+                const int d = (int)(mykey[j] >> KEY_POS_BITS);
+                const int u = (int)((unsigned)e_from[e] - smin), v = (int)((unsigned)e_to[e] - smin);
+                const int a0 = min_steps(s_loc, u, dmax, dmin), a1 = min_steps(v, e_loc, dmax, dmin);
+                atomicMin(&s_tlo[d], a0);
+                if (a1 <= L - 1) atomicMax(&s_thi[d], L - 1 - a1);
+            }
+        }
+        __syncthreads();
+        int2* tb = a.tband + goff;
+        for (int d = tid; d < DP; d += 1024) tb[d] = make_int2(s_tlo[d], s_thi[d]);
     }
 }
 
@@ -484,7 +539,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
 struct GatherArgs {
     const float* am; long long st_t, st_b;
     int T, B;
-    const SeqMeta* meta; const int* demis; float* gtab;
+    const SeqMeta* meta; const int* demis; const int2* tband; float* gtab;
     int* sync;
 };
 
@@ -502,12 +557,16 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
     float* g = a.gtab + (size_t)a.T * goff;
     const float* am = a.am + (long long)b * a.st_b;
     const int nt = min(TG, m.L - t0);
+    const int2* tb = a.tband + goff;
     for (int idx = threadIdx.x; idx < m.DP; idx += 256) {
         const int e = de[idx];
+        const int2 band = tb[idx];        // frames outside [band.x, band.y] get +inf without a read
         float v[TG];
 #pragma unroll
-        for (int tt = 0; tt < TG; tt++)
-            if (tt < nt) v[tt] = am[(long long)(t0 + tt) * a.st_t + e];
+        for (int tt = 0; tt < TG; tt++) {
+            v[tt] = INF_F;
+            if (tt < nt && t0 + tt >= band.x && t0 + tt <= band.y) v[tt] = am[(long long)(t0 + tt) * a.st_t + e];
+        }
 #pragma unroll
         for (int tt = 0; tt < TG; tt++)
             if (tt < nt) store_x<SYNC>(&g[(size_t)(t0 + tt) * m.DP + idx], v[tt] * LOG2E);
@@ -946,7 +1005,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     // sequence index fastest: workgroups that run together write neighbouring rows
     const int b = blockIdx.x, tid = threadIdx.x;
     const SeqMeta m = a.meta[b];
-    if (seq_error(m) || m.n_edges == 0 || m.L == 0) return;      // fbw_padfill writes those rows
+    if (m.L == 0) return;                                      // fbw_padfill has written every row
     const int T = a.T, B = a.B, F = a.F;
     // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
     // forward and the backward recursion meet, so those rows are complete first
@@ -954,7 +1013,17 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     if (y >= n) return;
     const int strip = (y & 1) ? n / 2 - 1 - (y >> 1) : n / 2 + (y >> 1);
     const int t0 = strip * TC;
-    const int tv = min(m.L, t0 + TC);    // frames [t0, tv) of this strip, all of them carry mass
+    const int tv = min(m.L, t0 + TC);    // frames [t0, tv) of this strip, all of them below seq_len
+    if (seq_error(m) || m.n_edges == 0) {
+        // no recursion ran for this sequence: NaN for a reported problem, empty frames otherwise
+        const bool err = seq_error(m) != 0;
+        const float v = err ? __builtin_nanf("") : (a.out_mode == I6FBW_OUT_PROB ? 0.f : INF_F);
+        for (int t = t0; t < tv; t++) {
+            stream_const_row(a.out + ((size_t)t * a.B + b) * a.F, a.F, v);
+            if (tid == 0) a.sum_output[(size_t)t * a.B + b] = err ? __builtin_nanf("") : 0.f;
+        }
+        return;
+    }
     if (SYNC) {
         // alpha rows [0, count_a) and beta rows [L - count_b, L) have been written through
         __shared__ int s_ok;
@@ -1128,20 +1197,20 @@ __global__ __launch_bounds__(64) void fbw_gate(int* sync, int need) {
     if (threadIdx.x == 0) spin_until_ge(sync + 1, need, sync);
 }
 
-// Rows that carry no probability mass: frames t >= seq_len, and every frame of a sequence without
-// edges, with seq_len outside [1, T] (out = hole, sum_output = 0: fbw_op.cu:120-128,366-369) or
-// with a reported problem (NaN).  These rows depend on nothing but the meta records.
-__global__ __launch_bounds__(COMB_THREADS) void fbw_padfill(CombArgs a) {
+// Rows of frames t >= seq_len (all rows if seq_len is outside [1, T]): out = hole, sum_output = 0
+// (fbw_op.cu:120-128,366-369).  They depend on nothing but seq_lens, so this kernel runs beside
+// the edge preparation.  Sequences that turn out to have no edges or a problem are written by
+// fbw_combine.
+__global__ __launch_bounds__(COMB_THREADS) void fbw_padfill(const int32_t* seq_lens, int T, int B, int F, int out_mode,
+                                                            float* out, float* sum_output) {
     const int b = blockIdx.x, t0 = blockIdx.y * TC;
-    const SeqMeta m = a.meta[b];
-    const int err = seq_error(m);
-    const int L = (err || m.n_edges == 0) ? 0 : m.L;
-    const int t1 = min(a.T, t0 + TC);
-    const float hole = a.out_mode == I6FBW_OUT_PROB ? 0.f : INF_F;
-    const float v = err ? __builtin_nanf("") : hole;
+    const unsigned sl = (unsigned)seq_lens[b];
+    const int L = (sl >= 1u && sl <= (unsigned)T) ? (int)sl : 0;
+    const int t1 = min(T, t0 + TC);
+    const float hole = out_mode == I6FBW_OUT_PROB ? 0.f : INF_F;
     for (int t = max(t0, L); t < t1; t++) {
-        stream_const_row(a.out + ((size_t)t * a.B + b) * a.F, a.F, v);
-        if (threadIdx.x == 0) a.sum_output[(size_t)t * a.B + b] = err ? __builtin_nanf("") : 0.f;
+        stream_const_row(out + ((size_t)t * B + b) * F, F, hole);
+        if (threadIdx.x == 0) sum_output[(size_t)t * B + b] = 0.f;
     }
 }
 
@@ -1166,7 +1235,7 @@ thread_local hipError_t g_last_hip_error = hipSuccess;
 struct Pipeline {
     bool ready = false;
     hipStream_t sG = nullptr, sC = nullptr;
-    hipEvent_t fork = nullptr, gathered = nullptr, join = nullptr;
+    hipEvent_t start = nullptr, fork = nullptr, gathered = nullptr, join = nullptr;
     int n_cu = 256;
 };
 Pipeline g_pipe[MAX_DEVICES];
@@ -1180,6 +1249,7 @@ int pipeline_init(Pipeline& p) {
     // default priority on purpose
     HIP_TRY(hipStreamCreateWithFlags(&p.sG, hipStreamNonBlocking));
     HIP_TRY(hipStreamCreateWithFlags(&p.sC, hipStreamNonBlocking));
+    HIP_TRY(hipEventCreateWithFlags(&p.start, hipEventDisableTiming));
     HIP_TRY(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
     HIP_TRY(hipEventCreateWithFlags(&p.gathered, hipEventDisableTiming));
     HIP_TRY(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
@@ -1268,13 +1338,24 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     hipStream_t sG = overlap ? P.sG : s, sC = overlap ? P.sC : s;
     if (g_prof.on) g_prof.n_calls++;
 
+    const dim3 g_grid(B, (T + TG - 1) / TG), c_grid(B, (T + TC - 1) / TC);
+    if (overlap) {
+        HIP_TRY(hipEventRecord(P.start, s));
+        HIP_TRY(hipStreamWaitEvent(sC, P.start, 0));
+    }
+    {   // rows of frames beyond seq_len depend on seq_lens only
+        StageTimer tm(4, sC);
+        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sC, seq_lens, T, B, F, out_mode, out, sum_output);
+        HIP_TRY(hipGetLastError());
+    }
+
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
     pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
-    pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis);
+    pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
     {
         StageTimer tm(0, s);
         if (E > 0) {
@@ -1288,7 +1369,7 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
 
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
-    ga.meta = meta; ga.demis = pa.demis; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
+    ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
     RecArgs ra;
     ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
@@ -1298,12 +1379,9 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
     ca.out = out; ca.sum_output = sum_output; ca.sync = sync;
-    const dim3 g_grid(B, (T + TG - 1) / TG), c_grid(B, (T + TC - 1) / TC);
     const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
     if (!overlap) {
-        { StageTimer tm(4, s); hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, s, ca); }
-        HIP_TRY(hipGetLastError());
         { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
         { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<false, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
@@ -1316,7 +1394,6 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
 
     HIP_TRY(hipEventRecord(P.fork, s));
     HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
-    HIP_TRY(hipStreamWaitEvent(sC, P.fork, 0));
     // Enqueue order gather -> recursion -> combine: every in-kernel wait is for a kernel enqueued
     // earlier, so the call also completes (without overlap) if the runtime maps two of the
     // streams onto one hardware queue.
@@ -1325,9 +1402,6 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     HIP_TRY(hipEventRecord(P.gathered, sG));
     { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
       else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
-    HIP_TRY(hipGetLastError());
-    // rows without probability mass depend on the meta records only
-    { StageTimer tm(4, sC); hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sC, ca); }
     HIP_TRY(hipGetLastError());
     // The dense write starts when the gather is done: by then the recursions are about to meet in
     // the middle of the sequences, which is where the combine kernel begins.
