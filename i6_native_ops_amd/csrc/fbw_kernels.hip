@@ -81,7 +81,7 @@ __host__ __device__ inline long long state_off(long long edge_begin, int b) { re
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 
 struct Layout {
-    size_t meta, sync, sortflag, eidx, ellA, ellB, crec, cbegin, demis, tband, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
 };
 
@@ -95,6 +95,7 @@ Layout make_layout(long long T, long long B, long long E) {
     l.meta = o;     o = align256(o + sizeof(SeqMeta) * B);
     l.sync = o;     o = align256(o + sizeof(int) * (SYNC_HDR + 2 * B + B * ((T + TG - 1) / TG)));
     l.sortflag = o; o = align256(o + sizeof(int) * (E / SCAN_BLOCK + 2));
+    l.seqbegin = o; o = align256(o + sizeof(int) * (B + 2));
     l.eidx = o;     o = align256(o + sizeof(int) * (E + 1));
     l.ellA = o;     o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
     l.ellB = o;     o = align256(o + sizeof(uint2) * KMAX * l.ss_total);
@@ -196,18 +197,29 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
-    SeqMeta* meta; int* sync; int* sortflag; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
+    SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
-// sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never decrease
-__global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int E, int* sortflag) {
+// sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never
+// decrease.  Where the index steps up, the first edge of every sequence in between is recorded:
+// seqbegin[q] = first edge with sequence index >= q (valid if the whole list turns out sorted).
+__global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int E, int B, int* sortflag, int* seqbegin) {
     __shared__ int bad;
     if (threadIdx.x == 0) bad = 0;
     __syncthreads();
     const int base = blockIdx.x * SCAN_BLOCK;
     int mybad = 0;
-    for (int i = base + threadIdx.x; i < min(E - 1, base + SCAN_BLOCK); i += 256)
-        mybad |= (unsigned)e_seq[i] > (unsigned)e_seq[i + 1];
+    for (int i = base + threadIdx.x; i < min(E, base + SCAN_BLOCK); i += 256) {
+        const unsigned cur = (unsigned)e_seq[i];
+        const unsigned prev = i > 0 ? (unsigned)e_seq[i - 1] : 0u;
+        mybad |= cur < prev;
+        // sequences prev+1 .. cur (from 0 for the first edge) start at edge i
+        unsigned q0 = i > 0 ? prev + 1u : 0u;
+        if (cur >= q0 && cur != 0xffffffffu)
+            for (unsigned q = q0; q <= min(cur, (unsigned)B); q++) seqbegin[q] = i;
+        if (i == E - 1)
+            for (unsigned q = min(cur, (unsigned)B) + 1u; q <= (unsigned)B; q++) seqbegin[q] = E;
+    }
     if (mybad) atomicOr(&bad, 1);
     __syncthreads();
     if (threadIdx.x == 0) sortflag[blockIdx.x] = !bad;
@@ -246,16 +258,6 @@ __device__ inline int lower_bound_hi(const unsigned* keys, int n, unsigned p) {
     }
     return lo;
 }
-// first index i in [0,n) with (unsigned)a[i] >= v, for a non-decreasing global array
-__device__ inline int lower_bound_u32(const int32_t* a, int n, unsigned v) {
-    int lo = 0, hi = n;
-    while (lo < hi) {
-        int mid = (lo + hi) >> 1;
-        if ((unsigned)a[mid] < v) lo = mid + 1; else hi = mid;
-    }
-    return lo;
-}
-
 // Lower bound on the number of edges of any path from state id `from` to state id `to` when no
 // edge raises the id by more than dmax or lowers it by more than -dmin.  Exact for left-to-right
 // chains numbered along the chain; never larger than the true distance for any automaton.
@@ -268,8 +270,8 @@ __device__ inline int min_steps(int from, int to, int dmax, int dmin) {
 
 // grid (3, B): role 0 orders the edges of sequence b by target state (alpha), role 1 by source
 // state (beta), role 2 by emission slot (combine) and writes the shared part of the meta record.
-// Edge lists grouped by sequence (the usual case) are located by binary search; any other order
-// is handled by a stable scan over the whole list.
+// For edge lists grouped by sequence (the usual case) the scan kernel has recorded where each
+// sequence starts; any other order is handled by a stable scan over the whole list.
 __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     __shared__ unsigned keys[EB_MAX];
     __shared__ unsigned bitmap[F_BITMAP_MAX / 32];
@@ -300,8 +302,8 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     const int chunk = (E + 1023) / 1024;
     const int lo = min(E, tid * chunk), hi = min(E, lo + chunk);
     if (sorted) {
-        edge_begin = lower_bound_u32(e_seq, E, (unsigned)b);
-        n_edges = lower_bound_u32(e_seq, E, (unsigned)b + 1u) - edge_begin;
+        edge_begin = E > 0 ? a.seqbegin[b] : 0;
+        n_edges = E > 0 ? a.seqbegin[b + 1] - edge_begin : 0;
         if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B) bad = 1;
         for (int i = edge_begin + tid; i < edge_begin + n_edges; i += 1024) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
@@ -1001,6 +1003,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
     static_assert(COMB_THREADS == 256, "block reductions assume 4 waves");
+    static_assert(TC == TG, "a combine strip waits for exactly one gather strip");
 
     // sequence index fastest: workgroups that run together write neighbouring rows
     const int b = blockIdx.x, tid = threadIdx.x;
@@ -1029,7 +1032,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
         __shared__ int s_ok;
         if (tid == 0) {
             const int* prog = a.sync + SYNC_HDR + 2 * b;
-            bool ok = spin_until_ge(prog, tv, a.sync);
+            // the gather strip of these frames (TC == TG, strips coincide), then both recursions
+            bool ok = spin_until_ge(a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG) + strip, 1, a.sync);
+            ok = ok && spin_until_ge(prog, tv, a.sync);
             ok = ok && spin_until_ge(prog + 1, m.L - t0, a.sync);
             s_ok = ok;
         }
@@ -1112,7 +1117,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             const float* grow = gbase + (size_t)t * DP;
 #pragma unroll
             for (int j = 0; j < JE; j++) {
-                va[j] = load_x<SYNC>(arow + efr[j]); vb[j] = load_x<SYNC>(brow + eto[j]); vg[j] = grow[esl[j]];
+                va[j] = load_x<SYNC>(arow + efr[j]); vb[j] = load_x<SYNC>(brow + eto[j]); vg[j] = load_x<SYNC>(grow + esl[j]);
             }
             if (tid == 0) voff = load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t);
         };
@@ -1151,7 +1156,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             const float* grow = gbase + (size_t)t * DP;
             auto score = [&](int i) {
                 const uint4 r = crec[i];
-                return (load_x<SYNC>(arow + (r.x & 0xFFFFu)) + __uint_as_float(r.y)) + (grow[r.z] + load_x<SYNC>(brow + (r.x >> 16)));
+                return (load_x<SYNC>(arow + (r.x & 0xFFFFu)) + __uint_as_float(r.y)) + (load_x<SYNC>(grow + r.z) + load_x<SYNC>(brow + (r.x >> 16)));
             };
             float lmin = INF_F;
             for (int i = tid; i < nE; i += COMB_THREADS) lmin = fminf(lmin, score(i));
@@ -1228,14 +1233,14 @@ thread_local hipError_t g_last_hip_error = hipSuccess;
         if (e_ != hipSuccess) { g_last_hip_error = e_; return I6FBW_ERR_LAUNCH; } \
     } while (0)
 
-// Library-owned streams and events of one device.  A large call forks from the caller's stream
-// after the edge preparation: the recursion stays on the caller's stream, the gather runs beside
-// it on a second stream and feeds it through flags in memory, and the dense write runs on a
-// third stream, started when the gather is done and fed by the recursion's progress counters.
+// Library-owned streams and events of one device.  A large call keeps the edge preparation and
+// the dense write (the first and the last kernel) on the caller's stream and runs the padding
+// fill, the gather and the recursion beside them on three streams of its own; the kernels that run
+// at the same time feed each other through flags in memory.
 struct Pipeline {
     bool ready = false;
-    hipStream_t sG = nullptr, sC = nullptr;
-    hipEvent_t start = nullptr, fork = nullptr, gathered = nullptr, join = nullptr;
+    hipStream_t sP = nullptr, sG = nullptr, sR = nullptr;
+    hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneG = nullptr, doneR = nullptr;
     int n_cu = 256;
 };
 Pipeline g_pipe[MAX_DEVICES];
@@ -1247,12 +1252,11 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipGetDevice(&dev));
     HIP_TRY(hipDeviceGetAttribute(&p.n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     // default priority on purpose
+    HIP_TRY(hipStreamCreateWithFlags(&p.sP, hipStreamNonBlocking));
     HIP_TRY(hipStreamCreateWithFlags(&p.sG, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&p.sC, hipStreamNonBlocking));
-    HIP_TRY(hipEventCreateWithFlags(&p.start, hipEventDisableTiming));
-    HIP_TRY(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
-    HIP_TRY(hipEventCreateWithFlags(&p.gathered, hipEventDisableTiming));
-    HIP_TRY(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
+    HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
+    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneG, &p.doneR})
+        HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     p.ready = true;
@@ -1335,32 +1339,33 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
     const int forced = g_overlap_mode;
     const bool overlap = forced >= 0 ? forced != 0 : (long long)T * B * F >= (1LL << 26);
-    hipStream_t sG = overlap ? P.sG : s, sC = overlap ? P.sC : s;
+    hipStream_t sP = overlap ? P.sP : s, sG = overlap ? P.sG : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;
 
     const dim3 g_grid(B, (T + TG - 1) / TG), c_grid(B, (T + TC - 1) / TC);
     if (overlap) {
         HIP_TRY(hipEventRecord(P.start, s));
-        HIP_TRY(hipStreamWaitEvent(sC, P.start, 0));
+        HIP_TRY(hipStreamWaitEvent(sP, P.start, 0));
     }
     {   // rows of frames beyond seq_len depend on seq_lens only
-        StageTimer tm(4, sC);
-        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sC, seq_lens, T, B, F, out_mode, out, sum_output);
+        StageTimer tm(4, sP);
+        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, sum_output);
         HIP_TRY(hipGetLastError());
     }
+    if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
 
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
     pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states;
-    pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.eidx = (int*)(ws + l.eidx);
+    pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
     {
         StageTimer tm(0, s);
         if (E > 0) {
             hipLaunchKernelGGL(fbw_scan_sorted, dim3((E + SCAN_BLOCK - 1) / SCAN_BLOCK), dim3(256), 0, s,
-                               edges + 3 * edge_row_stride, E, pa.sortflag);
+                               edges + 3 * edge_row_stride, E, B, pa.sortflag, pa.seqbegin);
             HIP_TRY(hipGetLastError());
         }
         hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
@@ -1394,24 +1399,30 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
 
     HIP_TRY(hipEventRecord(P.fork, s));
     HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
+    HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
     // Enqueue order gather -> recursion -> combine: every in-kernel wait is for a kernel enqueued
     // earlier, so the call also completes (without overlap) if the runtime maps two of the
     // streams onto one hardware queue.
     { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipEventRecord(P.gathered, sG));
-    { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
-      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
+    HIP_TRY(hipEventRecord(P.doneG, sG));
+    { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
+      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
     HIP_TRY(hipGetLastError());
-    // The dense write starts when the gather is done: by then the recursions are about to meet in
-    // the middle of the sequences, which is where the combine kernel begins.
-    HIP_TRY(hipStreamWaitEvent(sC, P.gathered, 0));
-    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sC, sync, 2 * B);
+    HIP_TRY(hipEventRecord(P.doneR, sR));
+    // The dense write is the last kernel on the caller's stream.  It starts when the gather is
+    // done (its workgroups would only take wave slots away from the gather before that: by then the
+    // two recursions are about to meet in the middle of the sequences, where the dense write
+    // begins) and the gate has seen every recursion workgroup on the machine; from then on each
+    // of its workgroups waits for the recursion progress it needs.
+    HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
+    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
     HIP_TRY(hipGetLastError());
-    { StageTimer tm(3, sC); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), sC, ca); }
+    { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipEventRecord(P.join, sC));
-    HIP_TRY(hipStreamWaitEvent(s, P.join, 0));
+    // join: all three finish well before the dense write does
+    HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
+    HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     return I6FBW_OK;
 }
 
