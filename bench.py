@@ -33,6 +33,9 @@ def main():
     ap.add_argument("--workload", default="cart", help="tiny | monophone | cart | ctc | longform")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--out-mode", type=int, default=1, help="0: -log posterior with +inf holes, 1: posterior")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain elementwise copy kernel over 1 GiB (3 times) so that a rocprofv3 --pmc run of "
+                         "this command shows what FETCH_SIZE / WRITE_SIZE read for a known amount of traffic")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU only (sequences are independent; sharding the batch over "
@@ -67,6 +70,14 @@ def main():
                  start_end.data_ptr(), start_end.stride(0), seq_lens.data_ptr(), W.T, W.B, W.F, W.E, W.n_states,
                  args.out_mode, out.data_ptr(), loss.data_ptr(), ws.data_ptr(), ws_bytes, stream)
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)      # an elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
     step()
     code, seq = cabi.read_status(ws.data_ptr(), W.B, stream)
     if code != 0:
@@ -100,11 +111,15 @@ def main():
     comb_bytes = (4 * W.F + 4) * W.seq_frames()
     comb_ms = stage_ms[3]
     comb_gbps = comb_bytes / (comb_ms * 1e-3) / 1e9 if comb_ms > 0 else 0.0
+    # HBM bytes per call of the dominant kernel, from the committed rocprofv3 --pmc summary
+    # (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for a copy kernel of known size)
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    tpath = os.path.join(ROOT, "profiles", f"fbw_{args.workload}_hbm_traffic.txt")
     if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get(args.workload, {}).get("combine_hbm_bytes")
+        import re
+        m = re.search(r"fbw_combine, scaled:.*= ([0-9.]+) MB per launch", open(tpath).read())
+        if m:
+            traffic = int(float(m.group(1)) * 1e6)
 
     result = {
         "metric": "FBW loss+grad ms/call + achieved HBM GB/s at T=1000,B=32,F=12001 fp32",
