@@ -41,7 +41,16 @@ constexpr int D_MAX = 4096;           // distinct emissions of one sequence
 #define I6_GATHER_BFAST 0
 #endif
 constexpr int TG = I6_TG;             // frames per gather workgroup
-constexpr int TC = 8;                 // frames per combine workgroup
+#ifndef I6_P1
+#define I6_P1 8
+#endif
+#ifndef I6_REC_PAD_LDS
+#define I6_REC_PAD_LDS 0
+#endif
+#ifndef I6_TC
+#define I6_TC 8
+#endif
+constexpr int TC = I6_TC;             // frames per combine workgroup
 constexpr int RENORM = 8;             // frames between renormalisations of the state vector
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
@@ -111,6 +120,10 @@ Layout make_layout(long long T, long long B, long long E) {
     l.total = o;
     return l;
 }
+
+#ifdef I6_TRACE
+__device__ unsigned long long g_trace[4096];   // debug builds only: in-kernel timestamps
+#endif
 
 // ---------------------------------------------------------------------------------------------
 // small device helpers
@@ -578,6 +591,9 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
         __syncthreads();
         if (threadIdx.x == 0) store_agent(&a.sync[SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG) + j], 1);
     }
+#ifdef I6_TRACE
+    if (threadIdx.x == 0) { atomicMax(&g_trace[1], wall_clock64()); atomicMin(&g_trace[0], wall_clock64()); if (b == 0) g_trace[512 + j] = wall_clock64(); }
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -614,6 +630,9 @@ struct RecCursor {
 // would cost several microseconds per publication while the dense write saturates the memory.
 template <bool SYNC>
 __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
+#ifdef I6_TRACE
+    if (threadIdx.x == 0 && (i % 50) == 0 && blockIdx.x < 4) g_trace[64 + blockIdx.x * 64 + i / 50] = wall_clock64();
+#endif
     static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
     const bool last = i + 1 == cur.nsteps;
     const bool pub = SYNC && (((i + 1) % PUBLISH) == 0 || last);
@@ -659,7 +678,11 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
         const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
         stn[s] = r;
+#ifdef I6_HACK_SPARSE_STORES
+        if (s < SP && (i & 3) == 0) store_x<SYNC>(cur.wp + s, r);
+#else
         if (s < SP) store_x<SYNC>(cur.wp + s, r);
+#endif
         rmin = fminf(rmin, r);
     }
     if (tid == 0) store_x<SYNC>(cur.op, cur.c);
@@ -885,6 +908,9 @@ __global__ __launch_bounds__(REC_BLOCK, DENSE ? 5 : 1) void fbw_recurse(RecArgs 
     __shared__ __attribute__((aligned(16))) float amr[2][D_MAX];
     __shared__ float wmin[NW];
 
+    // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
+    // gather or combine waves
+    __builtin_amdgcn_s_setprio(3);
     // every workgroup reports that it has been placed (see fbw_gate)
     if (SYNC && threadIdx.x == 0) atomicAdd(&a.sync[1], 1);
     const int b = blockIdx.x >> 1, dir = blockIdx.x & 1;
@@ -896,7 +922,7 @@ __global__ __launch_bounds__(REC_BLOCK, DENSE ? 5 : 1) void fbw_recurse(RecArgs 
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     if (cls == 1) {
-        if (loader) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
+        if (loader) recurse_load<SYNC, T_, 4, (DENSE ? 8 : I6_P1)>(a, m, b, dir, amr[0], amr[1]);
         else if (K <= 2) recurse_compute<SYNC, T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
@@ -1003,7 +1029,6 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
     static_assert(COMB_THREADS == 256, "block reductions assume 4 waves");
-    static_assert(TC == TG, "a combine strip waits for exactly one gather strip");
 
     // sequence index fastest: workgroups that run together write neighbouring rows
     const int b = blockIdx.x, tid = threadIdx.x;
@@ -1017,6 +1042,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     const int strip = (y & 1) ? n / 2 - 1 - (y >> 1) : n / 2 + (y >> 1);
     const int t0 = strip * TC;
     const int tv = min(m.L, t0 + TC);    // frames [t0, tv) of this strip, all of them below seq_len
+#ifdef I6_TRACE
+    if (tid == 0) { atomicMin(&g_trace[2], wall_clock64()); if (b == 0) g_trace[1024 + strip] = wall_clock64(); }
+#endif
     if (seq_error(m) || m.n_edges == 0) {
         // no recursion ran for this sequence: NaN for a reported problem, empty frames otherwise
         const bool err = seq_error(m) != 0;
@@ -1032,8 +1060,10 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
         __shared__ int s_ok;
         if (tid == 0) {
             const int* prog = a.sync + SYNC_HDR + 2 * b;
-            // the gather strip of these frames (TC == TG, strips coincide), then both recursions
-            bool ok = spin_until_ge(a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG) + strip, 1, a.sync);
+            // the gather strips of these frames, then both recursions
+            bool ok = true;
+            const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG);
+            for (int g = t0 / TG; ok && g <= (tv - 1) / TG; g++) ok = spin_until_ge(gflag + g, 1, a.sync);
             ok = ok && spin_until_ge(prog, tv, a.sync);
             ok = ok && spin_until_ge(prog + 1, m.L - t0, a.sync);
             s_ok = ok;
@@ -1195,6 +1225,17 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     }
 }
 
+// One-time check that two library streams really run at the same time (see pipeline_init).
+__device__ int g_selftest[4];
+__global__ void fbw_selftest_wait() {
+    if (threadIdx.x == 0) {
+        int seen = 0;
+        for (int n = 0; n < (1 << 18) && !seen; n++) { seen = load_agent(&g_selftest[0]); __builtin_amdgcn_s_sleep(8); }
+        store_agent(&g_selftest[1], seen ? 1 : 2);
+    }
+}
+__global__ void fbw_selftest_set(int v) { if (threadIdx.x == 0) store_agent(&g_selftest[0], v); }
+
 // Holds back the combine kernel (next on the same stream) until every workgroup of the recursion
 // kernel has been placed on the machine: combine workgroups wait for recursion progress while
 // they occupy LDS and wave slots, so they must not be able to keep a recursion workgroup out.
@@ -1242,6 +1283,7 @@ struct Pipeline {
     hipStream_t sP = nullptr, sG = nullptr, sR = nullptr;
     hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneG = nullptr, doneR = nullptr;
     int n_cu = 256;
+    bool concurrent = false;     // the recursion and gather streams were seen running at the same time
 };
 Pipeline g_pipe[MAX_DEVICES];
 std::mutex g_mutex;
@@ -1257,8 +1299,22 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
     for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneG, &p.doneR})
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 90 * 1024));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    // The overlapped schedule enqueues the recursion before the gather it waits for (so that its
+    // workgroups are placed at once).  That only works if the two streams are served at the same
+    // time; check it once with a bounded handshake and fall back to the single-stream schedule if
+    // the waiter never sees the flag (e.g. both streams mapped to one hardware queue).
+    fbw_selftest_set<<<1, 64, 0, p.sG>>>(0);
+    HIP_TRY(hipStreamSynchronize(p.sG));
+    fbw_selftest_wait<<<1, 64, 0, p.sR>>>();
+    fbw_selftest_set<<<1, 64, 0, p.sG>>>(1);
+    HIP_TRY(hipStreamSynchronize(p.sR));
+    HIP_TRY(hipStreamSynchronize(p.sG));
+    int result[4] = {0, 0, 0, 0};
+    HIP_TRY(hipMemcpyFromSymbol(result, HIP_SYMBOL(g_selftest), sizeof(result)));
+    p.concurrent = result[1] == 1;
     p.ready = true;
     return I6FBW_OK;
 }
@@ -1338,7 +1394,7 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     int* sync = (int*)(ws + l.sync);
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
     const int forced = g_overlap_mode;
-    const bool overlap = forced >= 0 ? forced != 0 : (long long)T * B * F >= (1LL << 26);
+    const bool overlap = P.concurrent && (forced >= 0 ? forced != 0 : (long long)T * B * F >= (1LL << 26));
     hipStream_t sP = overlap ? P.sP : s, sG = overlap ? P.sG : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;
 
@@ -1400,16 +1456,16 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     HIP_TRY(hipEventRecord(P.fork, s));
     HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
     HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
-    // Enqueue order gather -> recursion -> combine: every in-kernel wait is for a kernel enqueued
-    // earlier, so the call also completes (without overlap) if the runtime maps two of the
-    // streams onto one hardware queue.
-    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
-    HIP_TRY(hipGetLastError());
-    HIP_TRY(hipEventRecord(P.doneG, sG));
+    // The recursion goes first so that its 2B workgroups are placed before the gather fills the
+    // machine; its loader waves wait for the gather's strip flags (pipeline_init has checked that
+    // the two streams run side by side).  Every other in-kernel wait is for a kernel enqueued earlier.
     { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
       else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(P.doneR, sR));
+    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventRecord(P.doneG, sG));
     // The dense write is the last kernel on the caller's stream.  It starts when the gather is
     // done (its workgroups would only take wave slots away from the gather before that: by then the
     // two recursions are about to meet in the middle of the sequences, where the dense write
@@ -1468,6 +1524,11 @@ void i6fbw_set_overlap(int mode) {
     std::lock_guard<std::mutex> lock(g_mutex);
     g_overlap_mode = mode < 0 ? -1 : (mode ? 1 : 0);
 }
+
+#ifdef I6_TRACE
+int i6fbw_debug_trace(void* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * n); }
+int i6fbw_debug_trace_set(const void* host, int n) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), host, sizeof(unsigned long long) * n); }
+#endif
 
 const char* i6fbw_last_hip_error(void) { return g_last_hip_error == hipSuccess ? "" : hipGetErrorString(g_last_hip_error); }
 
