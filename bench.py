@@ -32,6 +32,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cart", help="tiny | monophone | cart | ctc | longform")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-wrapper", action="store_true", help="skip the wrapper-level (fbw_loss + backward) timing")
     ap.add_argument("--out-mode", type=int, default=1, help="0: -log posterior with +inf holes, 1: posterior")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise copy kernel over 1 GiB (3 times) so that a rocprofv3 --pmc run of "
@@ -145,6 +146,27 @@ def main():
                      "unit": "GB/s", "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "algorithmic_bytes_per_call": comb_bytes, "kernel_ms_per_call": round(comb_ms, 4)},
     }
+
+    # wrapper level (informational): fbw_loss(log_probs[B,T,F]).sum().backward() with the fused front end
+    # and with the reference's literal neg/transpose/contiguous/exp chain around the same kernels
+    if not args.no_wrapper:
+        from i6_native_ops_amd.fbw import fbw_loss, fbw_loss_unfused
+        fsa = (W.n_states, edges, weights, start_end)
+        base = am.neg().transpose(0, 1).contiguous()
+        wl = {}
+        for name, fn in (("fused_ms", fbw_loss), ("unfused_ms", fbw_loss_unfused)):
+            lp = base.clone().requires_grad_(True)
+            for it in range(8):
+                if it == 3:
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                lp.grad = None
+                fn(lp, fsa, seq_lens).sum().backward()
+            torch.cuda.synchronize()
+            wl[name] = round((time.perf_counter() - t0) / 5 * 1e3, 4)
+            del lp
+        result["config"]["wrapper_level"] = wl
+        del base
 
     if not args.no_cpu_baseline:
         from oracle import fbw_oracle

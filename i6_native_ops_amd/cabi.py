@@ -12,11 +12,12 @@ LIB_PATH = os.path.join(_HERE, "fbw", "libi6fbw.so")
 
 OUT_NEG_LOG = 0
 OUT_PROB = 1
+OUT_NEG_PROB = 2
 N_STAGES = 5
 STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
-SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
+SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
            "i6fbw_set_overlap",
            "i6fbw_profile_enable", "i6fbw_profile_read")
 
@@ -36,6 +37,11 @@ def load():
                                   c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
                                   c.c_void_p, c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
         lib.i6fbw_run.restype = c.c_int
+        lib.i6fbw_run_strided.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_int, c.c_void_p, c.c_int64, c.c_void_p,
+                                          c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
+                                          c.c_int, c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t,
+                                          c.c_void_p]
+        lib.i6fbw_run_strided.restype = c.c_int
         lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
         lib.i6fbw_read_status.restype = c.c_int
         lib.i6fbw_strerror.argtypes = [c.c_int]
@@ -72,6 +78,17 @@ def run(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_pt
     rc = load().i6fbw_run(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr,
                           se_row_stride, seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, sum_ptr, ws_ptr,
                           ws_bytes, stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def run_strided(am_ptr, am_stride_t, am_stride_b, scores_are_log_probs, edges_ptr, edge_row_stride, weights_ptr,
+                start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, out_stride_t,
+                out_stride_b, sum_ptr, ws_ptr, ws_bytes, stream=0) -> None:
+    rc = load().i6fbw_run_strided(am_ptr, am_stride_t, am_stride_b, int(scores_are_log_probs), edges_ptr,
+                                  edge_row_stride, weights_ptr, start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E,
+                                  n_states, out_mode, out_ptr, out_stride_t, out_stride_b, sum_ptr, ws_ptr, ws_bytes,
+                                  stream)
     if rc != 0:
         raise FbwError(rc)
 

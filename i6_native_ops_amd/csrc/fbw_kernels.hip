@@ -556,6 +556,7 @@ struct GatherArgs {
     int T, B;
     const SeqMeta* meta; const int* demis; const int2* tband; float* gtab;
     int* sync;
+    float scale;      // log2(e) for -log scores, -log2(e) for log scores
 };
 
 template <bool SYNC>
@@ -584,7 +585,7 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
         }
 #pragma unroll
         for (int tt = 0; tt < TG; tt++)
-            if (tt < nt) store_x<SYNC>(&g[(size_t)(t0 + tt) * m.DP + idx], v[tt] * LOG2E);
+            if (tt < nt) store_x<SYNC>(&g[(size_t)(t0 + tt) * m.DP + idx], v[tt] == INF_F ? INF_F : v[tt] * a.scale);
     }
     if (SYNC) {
         wait_stores();
@@ -950,6 +951,7 @@ struct CombArgs {
     const SeqMeta* meta; const uint4* crec; const int* cbegin; const int* demis;
     const float* alpha; const float* beta; const float* gtab; const double* offA; const double* offB;
     float* out; float* sum_output;
+    long long ost_t, ost_b;      // element strides of out over frames and sequences
     int* sync;
 };
 
@@ -1048,9 +1050,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     if (seq_error(m) || m.n_edges == 0) {
         // no recursion ran for this sequence: NaN for a reported problem, empty frames otherwise
         const bool err = seq_error(m) != 0;
-        const float v = err ? __builtin_nanf("") : (a.out_mode == I6FBW_OUT_PROB ? 0.f : INF_F);
+        const float v = err ? __builtin_nanf("") : (a.out_mode != I6FBW_OUT_NEG_LOG ? 0.f : INF_F);
         for (int t = t0; t < tv; t++) {
-            stream_const_row(a.out + ((size_t)t * a.B + b) * a.F, a.F, v);
+            stream_const_row(a.out + t * a.ost_t + b * a.ost_b, a.F, v);
             if (tid == 0) a.sum_output[(size_t)t * a.B + b] = err ? __builtin_nanf("") : 0.f;
         }
         return;
@@ -1071,8 +1073,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
         __syncthreads();
         if (!s_ok) return;       // timed out: reported through the abort flag
     }
-    const bool prob = a.out_mode == I6FBW_OUT_PROB;
+    const bool prob = a.out_mode != I6FBW_OUT_NEG_LOG;
     const float hole = prob ? 0.f : INF_F;
+    const float psign = a.out_mode == I6FBW_OUT_NEG_PROB ? -1.f : 1.f;
 
     float* image = (float*)lds4;
     const int F4 = (F + 32 + 3) >> 2;     // the image is shifted by the row's offset within its 128-byte line
@@ -1097,8 +1100,8 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
         const float logtot = __builtin_amdgcn_logf(tot);
         if (tid == 0)
             a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)(((double)(mn - logtot) + offs) * (double)LN2);
-        const float inv = dead ? 0.f : 1.f / tot;
-        float* orow = a.out + ((size_t)t * B + b) * F;
+        const float inv = dead ? 0.f : psign / tot;
+        float* orow = a.out + t * a.ost_t + b * a.ost_b;
         const int sh = row_misalign(orow);
         if (a_prev >= 0 && a_prev != sh) {
             for (int js = 0; js < nslot_regs; js++)
@@ -1248,14 +1251,14 @@ __global__ __launch_bounds__(64) void fbw_gate(int* sync, int need) {
 // the edge preparation.  Sequences that turn out to have no edges or a problem are written by
 // fbw_combine.
 __global__ __launch_bounds__(COMB_THREADS) void fbw_padfill(const int32_t* seq_lens, int T, int B, int F, int out_mode,
-                                                            float* out, float* sum_output) {
+                                                            float* out, long long ost_t, long long ost_b, float* sum_output) {
     const int b = blockIdx.x, t0 = blockIdx.y * TC;
     const unsigned sl = (unsigned)seq_lens[b];
     const int L = (sl >= 1u && sl <= (unsigned)T) ? (int)sl : 0;
     const int t1 = min(T, t0 + TC);
-    const float hole = out_mode == I6FBW_OUT_PROB ? 0.f : INF_F;
+    const float hole = out_mode != I6FBW_OUT_NEG_LOG ? 0.f : INF_F;
     for (int t = max(t0, L); t < t1; t++) {
-        stream_const_row(out + ((size_t)t * B + b) * F, F, hole);
+        stream_const_row(out + t * ost_t + b * ost_b, F, hole);
         if (threadIdx.x == 0) sum_output[(size_t)t * B + b] = 0.f;
     }
 }
@@ -1371,10 +1374,21 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
               const float* weights, const int32_t* start_end, int64_t se_row_stride, const int32_t* seq_lens, int T,
               int B, int F, int E, int n_states, int out_mode, float* out, float* sum_output, void* workspace,
               size_t workspace_bytes, void* stream_) {
+    return i6fbw_run_strided(am, am_stride_t, am_stride_b, 0, edges, edge_row_stride, weights, start_end, se_row_stride,
+                             seq_lens, T, B, F, E, n_states, out_mode, out, (int64_t)B * F, (int64_t)F, sum_output,
+                             workspace, workspace_bytes, stream_);
+}
+
+int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+                      const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
+                      int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
+                      int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
+                      void* workspace, size_t workspace_bytes, void* stream_) {
     if (T <= 0 || B <= 0 || F <= 0 || E < 0 || n_states <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (!am || !start_end || !seq_lens || !out || !sum_output || !workspace) return I6FBW_ERR_INVALID_ARGUMENT;
     if (E > 0 && (!edges || !weights)) return I6FBW_ERR_INVALID_ARGUMENT;
-    if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB && out_mode != I6FBW_OUT_NEG_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (out_stride_t < 0 || out_stride_b < 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
     const Layout l = make_layout(T, B, E);
@@ -1405,7 +1419,8 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     }
     {   // rows of frames beyond seq_len depend on seq_lens only
         StageTimer tm(4, sP);
-        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, sum_output);
+        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
+                           (long long)out_stride_b, sum_output);
         HIP_TRY(hipGetLastError());
     }
     if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
@@ -1431,6 +1446,7 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
+    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E;
     RecArgs ra;
     ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
@@ -1439,7 +1455,7 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
     ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
-    ca.out = out; ca.sum_output = sum_output; ca.sync = sync;
+    ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
     if (!overlap) {

@@ -40,41 +40,52 @@ static bool status_check_enabled() {
     return on;
 }
 
+// fused == false: am_scores is (T, B, F), -log p, contiguous; out is (T, B, F).
+// fused == true:  am_scores is log_probs (B, T, F) with unit innermost stride; out is (B, T, F).
 static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
                                       torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
-                                      int out_mode) {
-    CHECK_INPUT(am_scores, torch::kFloat32);
+                                      int out_mode, bool fused = false) {
+    if (fused) {
+        CHECK_CUDA(am_scores);
+        CHECK_TYPE(am_scores, torch::kFloat32);
+        TORCH_CHECK(am_scores.dim() == 3 && am_scores.stride(2) == 1, "log_probs must have shape (B, T, F) with unit innermost stride");
+    } else {
+        CHECK_INPUT(am_scores, torch::kFloat32);
+    }
     CHECK_INPUT(edges, torch::kInt32);
     CHECK_INPUT(weights, torch::kFloat32);
     CHECK_INPUT(start_end_states, torch::kInt32);
     CHECK_INPUT(seq_lens, torch::kInt32);
     // shape relations the reference asserts (fbw_op.cu:234-241,278-279)
     TORCH_CHECK(am_scores.dim() == 3, "am_scores must have shape (T, B, F)");
+    const int dt = fused ? 1 : 0, db = fused ? 0 : 1;      // which dimension is time / batch
     TORCH_CHECK(edges.dim() == 2 && edges.size(0) == 4, "edges must have shape (4, E)");
     TORCH_CHECK(weights.dim() == 1 && weights.size(0) == edges.size(1), "weights must have shape (E,)");
     TORCH_CHECK(start_end_states.dim() == 2 && start_end_states.size(0) == 2 &&
-                    start_end_states.size(1) == am_scores.size(1),
+                    start_end_states.size(1) == am_scores.size(db),
                 "start_end_states must have shape (2, B)");
-    TORCH_CHECK(seq_lens.dim() == 1 && seq_lens.size(0) == am_scores.size(1), "seq_lens must have shape (B,)");
+    TORCH_CHECK(seq_lens.dim() == 1 && seq_lens.size(0) == am_scores.size(db), "seq_lens must have shape (B,)");
     TORCH_CHECK(am_scores.size(0) > 0 && am_scores.size(1) > 0 && am_scores.size(2) > 0 && num_states > 0,
                 "NativeOp assertion failed: n_frames > 0, n_states > 0");
-    const int T = (int)am_scores.size(0), B = (int)am_scores.size(1), F = (int)am_scores.size(2);
+    const int T = (int)am_scores.size(dt), B = (int)am_scores.size(db), F = (int)am_scores.size(2);
     const int E = (int)edges.size(1);
 
     // PyTorch-ROCm presents HIP devices under the device type "cuda"
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(am_scores.device());
     auto opts = torch::TensorOptions().device(am_scores.device());
-    torch::Tensor out = torch::empty_like(am_scores);
+    torch::Tensor out = torch::empty(am_scores.sizes(), opts.dtype(torch::kFloat32));      // contiguous, same shape
     torch::Tensor sum_output = torch::empty({T, B}, opts.dtype(torch::kFloat32));
     size_t ws_bytes = 0;
     int rc = i6fbw_workspace_size(T, B, F, E, (int)num_states, &ws_bytes);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc));
     torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, opts.dtype(torch::kUInt8));
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
-    rc = i6fbw_run(am_scores.data_ptr<float>(), am_scores.stride(0), am_scores.stride(1), edges.data_ptr<int32_t>(),
-                   edges.stride(0), weights.data_ptr<float>(), start_end_states.data_ptr<int32_t>(),
-                   start_end_states.stride(0), seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode,
-                   out.data_ptr<float>(), sum_output.data_ptr<float>(), workspace.data_ptr(), ws_bytes, (void*)stream);
+    rc = i6fbw_run_strided(am_scores.data_ptr<float>(), am_scores.stride(dt), am_scores.stride(db), fused ? 1 : 0,
+                           edges.data_ptr<int32_t>(), edges.stride(0), weights.data_ptr<float>(),
+                           start_end_states.data_ptr<int32_t>(), start_end_states.stride(0),
+                           seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode, out.data_ptr<float>(),
+                           out.stride(dt), out.stride(db), sum_output.data_ptr<float>(), workspace.data_ptr(), ws_bytes,
+                           (void*)stream);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
     if (status_check_enabled()) {
         int code = 0, seq = -1;
@@ -98,6 +109,14 @@ std::vector<torch::Tensor> fbw_posterior(torch::Tensor& am_scores, torch::Tensor
     return run(am_scores, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_PROB);
 }
 
+// The whole of fbw_loss in one call: log_probs (B, T, F) in, [-posterior (B, T, F), loss (T, B)] out.
+// -posterior is what autograd delivers to log_probs through the reference wrapper's
+// neg().transpose(0, 1).contiguous() (fbw/__init__.py:66) and backward (fbw/__init__.py:40-44).
+std::vector<torch::Tensor> fbw_fused(torch::Tensor& log_probs, torch::Tensor& edges, torch::Tensor& weights,
+                                     torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states) {
+    return run(log_probs, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_NEG_PROB, true);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     py::class_<DebugOptions>(m, "DebugOptions")
         .def(py::init<>())
@@ -109,6 +128,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fbw", &fbw, "Fast Baum-Welch routine (MI355X)", py::arg("am_scores"), py::arg("edges"), py::arg("weights"),
           py::arg("start_end_states"), py::arg("seq_lens"), py::arg("num_states"),
           py::arg("debug_options") = DebugOptions());
+    m.def("fbw_fused", &fbw_fused,
+          "fbw_loss in one call: log_probs (B, T, F) -> [gradient w.r.t. log_probs = -posterior (B, T, F), loss (T, B)]");
     m.def("fbw_posterior", &fbw_posterior,
           "Same as fbw but the first result holds the posteriors themselves (exp(-out)) with 0 in the holes");
 }

@@ -42,6 +42,27 @@ class FastBaumWelchLoss(torch.autograd.Function):
         return ctx.saved_tensors[0], None, None
 
 
+class _FusedFbwLoss(torch.autograd.Function):
+    """fbw_loss without the wrapper's dense passes: the kernels read ``log_probs`` (B, T, F) in place
+    (sign flip and strides inside the gather) and write the gradient w.r.t. ``log_probs``, minus
+    the posteriors, in (B, T, F).  Same values as FastBaumWelchLoss behind the reference's
+    neg/transpose/contiguous chain (fbw/__init__.py:40-44,66), including the ignored grad_loss."""
+
+    @staticmethod
+    def forward(ctx, log_probs, fsa, seq_lens):
+        num_states, edge_tensor, weight_tensor, start_end_states = fsa
+        if log_probs.stride(-1) != 1:
+            log_probs = log_probs.contiguous()
+        grad, loss = core.fbw_fused(log_probs, edge_tensor, weight_tensor, start_end_states, seq_lens,
+                                    int(num_states))
+        ctx.save_for_backward(grad)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        return ctx.saved_tensors[0], None, None
+
+
 def fbw_loss(
     log_probs: torch.FloatTensor,
     fsa: Tuple[int, torch.IntTensor, torch.FloatTensor, torch.IntTensor],
@@ -57,8 +78,14 @@ def fbw_loss(
     :return: (T, B) tensor; entry (t, b) is the loss of sequence b for t < seq_lens[b], else 0
         (the reference's docstring says (B,), its code returns (T, B): fbw/__init__.py:32-38)
     """
+    return _FusedFbwLoss.apply(log_probs, fsa, seq_lens)
+
+
+def fbw_loss_unfused(log_probs, fsa, seq_lens):
+    """The reference's literal wrapper (fbw/__init__.py:66-67): explicit negation and transposition in
+    front of FastBaumWelchLoss.  Kept for comparison; fbw_loss gives the same values faster."""
     neg_log_probs = log_probs.neg().transpose(0, 1).contiguous()  # [T, B, F]
     return FastBaumWelchLoss.apply(neg_log_probs, fsa, seq_lens)
 
 
-__all__ = ["fbw_loss", "FastBaumWelchLoss", "core"]
+__all__ = ["fbw_loss", "fbw_loss_unfused", "FastBaumWelchLoss", "core"]

@@ -38,8 +38,10 @@ enum {
 enum {
     I6FBW_OUT_NEG_LOG = 0,   /* -log posterior, +inf where nothing contributes: what fbw_core.fbw returns
                                 (fbw_op.cu:366-377,392) */
-    I6FBW_OUT_PROB = 1       /* posterior itself, 0 where nothing contributes: what
+    I6FBW_OUT_PROB = 1,      /* posterior itself, 0 where nothing contributes: what
                                 FastBaumWelchLoss.backward derives from it (fbw/__init__.py:40-44) */
+    I6FBW_OUT_NEG_PROB = 2   /* minus the posterior: the gradient that reaches `log_probs` in fbw_loss
+                                after autograd has undone its neg() (fbw/__init__.py:43,66) */
 };
 
 /*
@@ -83,6 +85,25 @@ int i6fbw_run(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
               int T, int B, int F, int E, int n_states, int out_mode,
               float* out, float* sum_output,
               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * i6fbw_run with explicit layouts, for a caller that holds the (B, T, F) log-probabilities of
+ * fbw_loss (fbw/__init__.py:47-68) and wants the gradient in the same layout without the
+ * reference wrapper's dense passes (neg, transpose().contiguous(), neg, exp and their autograd
+ * inverses: fbw/__init__.py:43,66):
+ *   scores_are_log_probs  0: am_scores holds -log p (as for i6fbw_run), 1: it holds log p
+ *   out_stride_t/_b       element strides of out over frames / sequences (innermost stride 1);
+ *                         rows may overlap nothing else and need not be aligned
+ * i6fbw_run(...) is i6fbw_run_strided(..., 0, ..., out, B*F, F, ...).
+ */
+int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+                      const int32_t* edges, int64_t edge_row_stride,
+                      const float* weights,
+                      const int32_t* start_end, int64_t se_row_stride,
+                      const int32_t* seq_lens,
+                      int T, int B, int F, int E, int n_states, int out_mode,
+                      float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Waits for `stream` and copies the device-side status of the last i6fbw_run that

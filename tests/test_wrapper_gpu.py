@@ -117,3 +117,44 @@ def test_device_side_status_is_reported():
     # the good input still works afterwards
     out, loss = core.fbw(am, edges, weights, se, seq_lens, n)
     assert torch.isfinite(loss).all()
+
+
+@pytest.mark.parametrize("name,kw", [("tiny", {}), ("monophone", dict(T=80, B=6, F=60, shuffle_edges=True)),
+                                     ("ctc", dict(T=40, B=8, F=50)), ("cart", dict(T=300, B=3, F=12001))])
+@pytest.mark.parametrize("overlap", [0, 1])
+def test_fused_fbw_loss_equals_unfused_wrapper_and_oracle(oracle, name, kw, overlap):
+    """fbw_loss reads log_probs (B,T,F) in place and writes -posterior in (B,T,F); the reference's
+    literal wrapper (neg, transpose, contiguous, exp) must give the same loss and gradient."""
+    from i6_native_ops_amd import cabi
+    from i6_native_ops_amd.fbw import fbw_loss, fbw_loss_unfused
+    cabi.set_overlap(overlap)
+    try:
+        W = make_workload(name, **kw)
+        dev = "cuda"
+        fsa = (W.n_states, torch.from_numpy(W.edges).to(dev), torch.from_numpy(W.weights).to(dev),
+               torch.from_numpy(W.start_end_states).to(dev))
+        seq_lens = torch.from_numpy(W.seq_lens).to(dev)
+        base = torch.from_numpy(-W.am_scores).transpose(0, 1).contiguous().to(dev)          # [B,T,F] log probs
+        results = []
+        for fn in (fbw_loss, fbw_loss_unfused):
+            lp = base.clone().requires_grad_(True)
+            loss = fn(lp, fsa, seq_lens)
+            loss.sum().backward()
+            results.append((loss.detach().cpu().numpy(), lp.grad.cpu().numpy()))
+        want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens,
+                                                W.n_states)
+        want_grad = -np.exp(-want_out.astype(np.float64)).transpose(1, 0, 2)               # [B,T,F]
+        for loss, grad in results:
+            assert loss.shape == (W.T, W.B) and grad.shape == (W.B, W.T, W.F)
+            np.testing.assert_allclose(loss, want_loss, rtol=1e-5, atol=1e-6)
+            np.testing.assert_allclose(grad, want_grad, atol=1e-4)
+        np.testing.assert_allclose(results[0][0], results[1][0], rtol=1e-6)
+        np.testing.assert_allclose(results[0][1], results[1][1], atol=2e-6)
+        # a non-contiguous view with unit innermost stride is read in place
+        wide = torch.zeros(W.B, W.T, W.F + 5, device=dev)
+        wide[:, :, :W.F] = base
+        lp = wide[:, :, :W.F].requires_grad_(True)
+        loss = fbw_loss(lp, fsa, seq_lens)
+        np.testing.assert_array_equal(loss.detach().cpu().numpy(), results[0][0])
+    finally:
+        cabi.set_overlap(-1)
