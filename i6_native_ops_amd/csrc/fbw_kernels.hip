@@ -23,6 +23,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "../../include/i6fbw.h"
@@ -168,6 +169,19 @@ __device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort
     }
     atomicOr(abort_flag, 1);
     return false;
+}
+
+// Order in which gather and combine workgroups are handed out (1-D grid, dispatched in index
+// order): the batch is cut into `groups` blocks of `per_group` sequences, and a block goes through
+// all of its strips before the next block starts.  The first block's recursions then reach the
+// middle of their sequences, where the dense write can begin, after 1/groups of the gather, and
+// the gather of the later blocks runs beside the dense write of the earlier ones.
+__device__ __forceinline__ void grouped_index(int per_group, int n_strips, int B, int* b, int* y) {
+    const int bi = blockIdx.x % per_group;
+    const int rest = blockIdx.x / per_group;
+    *y = rest % n_strips;
+    *b = (rest / n_strips) * per_group + bi;
+    if (*b >= B) *b = -1;
 }
 
 // wave-wide minimum in lane 63 (DPP row operations, no LDS traffic)
@@ -557,11 +571,14 @@ struct GatherArgs {
     const SeqMeta* meta; const int* demis; const int2* tband; float* gtab;
     int* sync;
     float scale;      // log2(e) for -log scores, -log2(e) for log scores
+    int per_group;    // sequences per block of the hand-out order
 };
 
 template <bool SYNC>
 __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
-    const int b = blockIdx.x, y = blockIdx.y;
+    int b, y;
+    grouped_index(a.per_group, (a.T + TG - 1) / TG, a.B, &b, &y);
+    if (b < 0) return;
     const SeqMeta m = a.meta[b];
     if (rec_class(m) <= 0) return;
     const int n = (m.L + TG - 1) / TG;
@@ -632,7 +649,8 @@ struct RecCursor {
 template <bool SYNC>
 __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
 #ifdef I6_TRACE
-    if (threadIdx.x == 0 && (i % 50) == 0 && blockIdx.x < 4) g_trace[64 + blockIdx.x * 64 + i / 50] = wall_clock64();
+    if (threadIdx.x == 0 && (i % 50) == 0 && (blockIdx.x < 2 || blockIdx.x >= gridDim.x - 2))
+        g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + i / 50] = wall_clock64();
 #endif
     static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
     const bool last = i + 1 == cur.nsteps;
@@ -847,14 +865,22 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     auto cc = [&](int jl) { return min(lane + jl * 64, npiece - 1); };
     int* abort_flag = a.sync;
     const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((T + TG - 1) / TG);
-    int strip_ok = -1;
-    // row consumed by step i (clamped to the steps that exist); waits for its strip first
+    const int nstrip = (L + TG - 1) / TG;
+    int strip_ok = -1;                  // strip known to be complete
+    int ahead_strip = -1, ahead_val = 0;   // flag of the strip after it, loaded while strip_ok is being consumed
+    // row consumed by step i (clamped to the steps that exist); makes sure its strip is complete.
+    // The flag of the following strip is requested a strip ahead, so that in the steady state the
+    // loader never sits in a memory round trip while the compute waves wait at the barrier.
     auto rowp = [&](int i) -> const u64* {
         const int ic = min(i, nsteps - 1);
         const int f = dir ? L - 1 - ic : ic;
         if (SYNC && f / TG != strip_ok) {
-            spin_until_ge(gflag + f / TG, 1, abort_flag);
-            strip_ok = f / TG;
+            const int j = f / TG;
+            if (!(j == ahead_strip && ahead_val >= 1)) spin_until_ge(gflag + j, 1, abort_flag);
+            strip_ok = j;
+            const int jn = dir ? j - 1 : j + 1;
+            ahead_strip = -1;
+            if (jn >= 0 && jn < nstrip) { ahead_strip = jn; ahead_val = load_agent(gflag + jn); }
         }
         return (const u64*)(G + (size_t)f * DP);
     };
@@ -953,6 +979,7 @@ struct CombArgs {
     float* out; float* sum_output;
     long long ost_t, ost_b;      // element strides of out over frames and sequences
     int* sync;
+    int per_group;               // sequences per block of the hand-out order
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1032,14 +1059,18 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     __shared__ float redsum[COMB_THREADS / 64];
     static_assert(COMB_THREADS == 256, "block reductions assume 4 waves");
 
-    // sequence index fastest: workgroups that run together write neighbouring rows
-    const int b = blockIdx.x, tid = threadIdx.x;
+    // within a block of sequences the sequence index runs fastest: workgroups that run together
+    // write neighbouring rows
+    const int tid = threadIdx.x;
+    int b, y;
+    grouped_index(a.per_group, (a.T + TC - 1) / TC, a.B, &b, &y);
+    if (b < 0) return;
     const SeqMeta m = a.meta[b];
     if (m.L == 0) return;                                      // fbw_padfill has written every row
     const int T = a.T, B = a.B, F = a.F;
     // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
     // forward and the backward recursion meet, so those rows are complete first
-    const int n = (m.L + TC - 1) / TC, y = blockIdx.y;
+    const int n = (m.L + TC - 1) / TC;
     if (y >= n) return;
     const int strip = (y & 1) ? n / 2 - 1 - (y >> 1) : n / 2 + (y >> 1);
     const int t0 = strip * TC;
@@ -1355,6 +1386,12 @@ struct StageTimer {
 size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
+int g_groups = [] {
+    // blocks of sequences in the overlapped schedule; more than one lets the dense write start before
+    // the gather is over, which measured slower (the kernels get in each other's way), so the default is 1
+    const char* e = getenv("I6FBW_GROUPS");
+    return e ? atoi(e) : 0;
+}();
 int g_overlap_mode = [] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
@@ -1412,19 +1449,12 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     hipStream_t sP = overlap ? P.sP : s, sG = overlap ? P.sG : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;
 
-    const dim3 g_grid(B, (T + TG - 1) / TG), c_grid(B, (T + TC - 1) / TC);
-    if (overlap) {
-        HIP_TRY(hipEventRecord(P.start, s));
-        HIP_TRY(hipStreamWaitEvent(sP, P.start, 0));
-    }
-    {   // rows of frames beyond seq_len depend on seq_lens only
-        StageTimer tm(4, sP);
-        hipLaunchKernelGGL(fbw_padfill, c_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
-                           (long long)out_stride_b, sum_output);
-        HIP_TRY(hipGetLastError());
-    }
-    if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
-
+    // blocks of sequences for the hand-out order of gather and combine (see grouped_index)
+    const int groups = overlap ? std::max(1, std::min(g_groups > 0 ? g_groups : 1, B / 8)) : 1;
+    const int per_group = (B + groups - 1) / groups;
+    const dim3 g_grid((unsigned)(per_group * groups) * ((T + TG - 1) / TG)), c_grid((unsigned)(per_group * groups) * ((T + TC - 1) / TC));
+    const dim3 p_grid(B, (T + TC - 1) / TC);
+    if ((long long)per_group * groups * ((T + TG - 1) / TG) > 0x7fffffffLL) return I6FBW_ERR_INVALID_ARGUMENT;
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
@@ -1439,14 +1469,27 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
                                edges + 3 * edge_row_stride, E, B, pa.sortflag, pa.seqbegin);
             HIP_TRY(hipGetLastError());
         }
+        if (overlap) HIP_TRY(hipEventRecord(P.start, s));      // releases the padding fill, see below
         hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
         HIP_TRY(hipGetLastError());
     }
+    // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
+    // leaves the memory system idle.  The fill is released when the scan kernel is done, i.e. when
+    // the preparation's large workgroups are being placed, so that its many small workgroups
+    // cannot keep them off the machine.
+    if (overlap) HIP_TRY(hipStreamWaitEvent(sP, P.start, 0));
+    {
+        StageTimer tm(4, sP);
+        hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
+                           (long long)out_stride_b, sum_output);
+        HIP_TRY(hipGetLastError());
+    }
+    if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
 
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
-    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E;
+    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.per_group = per_group;
     RecArgs ra;
     ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
@@ -1455,7 +1498,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
-    ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
+    ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync; ca.per_group = per_group;
     const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
     if (!overlap) {
@@ -1479,7 +1522,15 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
       else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(P.doneR, sR));
-    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, sG, ga); }
+    // A recursion workgroup needs ten free wave slots on one compute unit at once; a running grid of
+    // small workgroups refills every slot it frees, so the gather is held back until all recursion
+    // workgroups have been placed.
+    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sG, sync, 2 * B);
+    HIP_TRY(hipGetLastError());
+#ifndef I6_GATHER_LDS
+#define I6_GATHER_LDS 0
+#endif
+    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), I6_GATHER_LDS, sG, ga); }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipEventRecord(P.doneG, sG));
     // The dense write is the last kernel on the caller's stream.  It starts when the gather is
@@ -1487,13 +1538,17 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // two recursions are about to meet in the middle of the sequences, where the dense write
     // begins) and the gate has seen every recursion workgroup on the machine; from then on each
     // of its workgroups waits for the recursion progress it needs.
-    HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
+    if (groups == 1) HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
+#ifdef I6_TRACE
+    if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
+#endif
     hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
     HIP_TRY(hipGetLastError());
     { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
     HIP_TRY(hipGetLastError());
     // join: all three finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
+    HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     return I6FBW_OK;
 }
