@@ -1,5 +1,5 @@
 """Builds the native parts in-tree: libi6fbw.so (HIP kernels + C ABI, hipcc, gfx950) and the
-PyTorch-ROCm binding fbw_core (links libi6fbw.so).  Takes the place of the reference's
+PyTorch-ROCm bindings fbw_core and fast_viterbi_core (both link libi6fbw.so).  Takes the place of the reference's
 setup.py FBW entry (setup.py:29-33) and its import-time JIT fallback (fbw/__init__.py:10-24):
 nothing is compiled at import time, and nothing is hipified."""
 import os
@@ -29,27 +29,30 @@ def build_lib():
     return LIB
 
 
-def build_ext():
+def build_ext(name="fbw_core", source="fbw_torch.cpp", out_dir=None):
     import torch
     from torch.utils import cpp_extension
     inc = cpp_extension.include_paths()
     torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
-           "-DTORCH_EXTENSION_NAME=fbw_core", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-DTORCH_EXTENSION_NAME=" + name, "-DTORCH_API_INCLUDE_EXTENSION_H",
            f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
            "-I" + sysconfig.get_paths()["include"], "-I/opt/rocm/include"]
     cmd += ["-I" + p for p in inc]
-    cmd += [os.path.join(CSRC, "fbw_torch.cpp"), "-o", EXT,
+    out_dir = out_dir or OUT
+    ext = os.path.join(out_dir, name + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+    cmd += [os.path.join(CSRC, source), "-o", ext,
             "-L" + OUT, "-li6fbw", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
             "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
-            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-Wl,-rpath,/opt/rocm/lib", "-Wno-attributes"]
+            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/../fbw", "-Wl,-rpath," + torch_lib, "-Wl,-rpath,/opt/rocm/lib", "-Wno-attributes"]
     _run(cmd)
-    return EXT
+    return ext
 
 
 def build_all():
     build_lib()
     build_ext()
+    build_ext("fast_viterbi_core", "viterbi_torch.cpp", os.path.join(PKG, "fast_viterbi"))
 
 
 if __name__ == "__main__":

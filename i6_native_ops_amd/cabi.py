@@ -18,7 +18,7 @@ STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
-           "i6fbw_set_overlap",
+           "i6fbw_set_overlap", "i6fbw_viterbi",
            "i6fbw_profile_enable", "i6fbw_profile_read")
 
 _lib = None
@@ -42,6 +42,10 @@ def load():
                                           c.c_int, c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t,
                                           c.c_void_p]
         lib.i6fbw_run_strided.restype = c.c_int
+        lib.i6fbw_viterbi.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_int64, c.c_void_p, c.c_void_p,
+                                      c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
+                                      c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
+        lib.i6fbw_viterbi.restype = c.c_int
         lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
         lib.i6fbw_read_status.restype = c.c_int
         lib.i6fbw_strerror.argtypes = [c.c_int]
@@ -89,6 +93,16 @@ def run_strided(am_ptr, am_stride_t, am_stride_b, scores_are_log_probs, edges_pt
                                   edge_row_stride, weights_ptr, start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E,
                                   n_states, out_mode, out_ptr, out_stride_t, out_stride_b, sum_ptr, ws_ptr, ws_bytes,
                                   stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def viterbi(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr, se_row_stride,
+            seq_lens_ptr, T, B, F, E, n_states, align_ptr, align_stride_t, align_stride_b, scores_ptr, ws_ptr,
+            ws_bytes, stream=0) -> None:
+    rc = load().i6fbw_viterbi(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr,
+                              start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E, n_states, align_ptr,
+                              align_stride_t, align_stride_b, scores_ptr, ws_ptr, ws_bytes, stream)
     if rc != 0:
         raise FbwError(rc)
 

@@ -224,6 +224,7 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
+    int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
@@ -429,6 +430,12 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
         return;
     }
 
+    if (a.best_path && role == 1) {
+        if (tid == 0) { a.meta[b].Kout = 0; a.meta[b].errB = 0; }
+        return;
+    }
+    const float wscale = a.best_path ? 1.f : LOG2E;
+
     auto slot_of = [&](unsigned em) -> unsigned {
         return (unsigned)wordpfx[em >> 5] + (unsigned)__popc(bitmap[em >> 5] & ((1u << (em & 31)) - 1u));
     };
@@ -463,7 +470,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
 
     if (role < 2) {
         // ELL table: entry (k, s) = k-th edge (in input order) entering (role 0) / leaving (role 1)
-        // local state s, as {other state | slot << 16, weight * log2(e)}; unused entries point at
+        // local state s, as {other state | slot << 16, weight * log2(e) (best path: weight)}; unused entries point at
         // NO_STATE.
         uint2* ell = (role == 0 ? a.ellA : a.ellB) + (size_t)KMAX * soff;
         int kmax = 0;
@@ -488,7 +495,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
             int e = edge_at((int)(keys[i] & POS_MASK));
             unsigned other = (role == 0 ? (unsigned)e_from[e] : (unsigned)e_to[e]) - smin;
             unsigned slot = slot_of((unsigned)e_emis[e]);
-            ell[(size_t)k * SP + p] = make_uint2(other | (slot << 16), __float_as_uint(a.weights[e] * LOG2E));
+            ell[(size_t)k * SP + p] = make_uint2(other | (slot << 16), __float_as_uint(a.weights[e] * wscale));
         }
     } else {
         // combine order: edges sorted by slot; CSR begin per slot; list of distinct emission ids
@@ -1458,7 +1465,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
-    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states;
+    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
@@ -1627,3 +1634,5 @@ int i6fbw_profile_read(float* stage_ms) {
 }
 
 }  // extern "C"
+
+#include "viterbi_kernels.inc"

@@ -114,6 +114,37 @@ int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_st
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq);
 
 /*
+ * Best path (Viterbi alignment) on the same automaton description.  Replaces fast_viterbi_cuda
+ * (i6_native_ops/fast_viterbi/core.cu:179-275; binding fast_viterbi/binding.cpp:13-25).
+ *
+ *   am_scores   float [T,B,F] with element strides am_stride_t / am_stride_b, innermost stride 1;
+ *               scores that are MAXIMISED (log probabilities; core.cu:109 adds them to the edge
+ *               weight, core.cu:20-49 keeps the larger sum)
+ *   edges, weights, start_end, seq_lens, n_states: as for i6fbw_run
+ *   alignment   int32, element (t, b) at t * align_stride_t + b * align_stride_b: emission index
+ *               of the edge the best path takes in frame t; 0 in frames >= seq_lens[b] and where
+ *               the walk back from the end state finds no back-pointer (core.cu:145-177)
+ *   scores      float [B]: value of the end state after seq_lens[b] frames, -inf without a path
+ *               (core.cu:124-143)
+ *   workspace   as for i6fbw_run (i6fbw_workspace_size bytes)
+ *
+ * Values are computed in the reference's arithmetic, (previous + weight) + score in fp32, and
+ * ties go to the edge that comes first in the input, as the reference's compare-and-swap rule
+ * decides them, so alignment and scores equal the reference's bit for bit.  seq_lens[b] > T
+ * (undefined in the reference) is read as T.  One kernel chain on `stream`; per-sequence
+ * problems are reported by i6fbw_read_status, the affected sequences get score NaN and an
+ * all-zero alignment.
+ */
+int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
+                  const int32_t* edges, int64_t edge_row_stride,
+                  const float* weights,
+                  const int32_t* start_end, int64_t se_row_stride,
+                  const int32_t* seq_lens,
+                  int T, int B, int F, int E, int n_states,
+                  int32_t* alignment, int64_t align_stride_t, int64_t align_stride_b, float* scores,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Chooses how i6fbw_run schedules its stages: 0 one after the other on the caller's stream,
  * 1 overlapped (gather, recursion and dense write run at the same time on library streams and
  * hand frames to each other through flags in the workspace), -1 (default) overlapped for large

@@ -2,7 +2,8 @@
 
 Only tests/, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
 ``bench.py`` may import this module.  The arithmetic lives in
-``fbw_oracle.c`` (a restatement of i6_native_ops/fbw/fbw_op.cu:17-153,226-393).
+``fbw_oracle.c`` (a restatement of i6_native_ops/fbw/fbw_op.cu:17-153,226-393) and
+``viterbi_oracle.c`` (i6_native_ops/fast_viterbi/core.cu:20-177,209-264).
 """
 import ctypes
 import os
@@ -43,6 +44,8 @@ def _load():
             fn.argtypes = argt
             fn.restype = ctypes.c_int
         lib.fbw_oracle_max_threads.restype = ctypes.c_int
+        lib.viterbi_oracle_f32.argtypes = argt[:-3] + [ctypes.c_void_p, ctypes.c_void_p]
+        lib.viterbi_oracle_f32.restype = ctypes.c_int
         _lib = lib
     return _lib
 
@@ -79,3 +82,28 @@ def fbw_oracle(am_scores, edges, weights, start_end_states, seq_lens, n_states, 
     if rc != 0:
         raise RuntimeError(f"fbw oracle failed with status {rc}")
     return out, loss
+
+
+def viterbi_oracle(am_scores, edges, weights, start_end_states, seq_lens, n_states):
+    """Same contract as ``fast_viterbi_core.fast_viterbi`` (fast_viterbi/binding.cpp:13-25) on host arrays.
+
+    :param am_scores: float32 [T,B,F] scores that are *maximised* (log probabilities)
+    :return: (alignment int32 [T,B] of emission indices, 0 in frames without a path; scores float32 [B])
+    """
+    lib = _load()
+    am = np.ascontiguousarray(am_scores, dtype=np.float32)
+    ed = np.ascontiguousarray(edges, dtype=np.int32)
+    w = np.ascontiguousarray(weights, dtype=np.float32)
+    se = np.ascontiguousarray(start_end_states, dtype=np.int32)
+    sl = np.ascontiguousarray(seq_lens, dtype=np.int32)
+    T, B, F = am.shape
+    assert ed.ndim == 2 and ed.shape[0] == 4
+    E = ed.shape[1]
+    assert w.shape == (E,) and se.shape == (2, B) and sl.shape == (B,)
+    alignment = np.empty((T, B), dtype=np.int32)
+    scores = np.empty((B,), dtype=np.float32)
+    rc = lib.viterbi_oracle_f32(am.ctypes.data, B * F, F, ed.ctypes.data, E, w.ctypes.data, se.ctypes.data, B,
+                                sl.ctypes.data, T, B, F, E, int(n_states), alignment.ctypes.data, scores.ctypes.data)
+    if rc != 0:
+        raise RuntimeError(f"viterbi oracle failed with status {rc}")
+    return alignment, scores

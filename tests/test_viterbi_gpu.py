@@ -1,0 +1,150 @@
+"""Best-path alignment on the GPU against the oracle: alignment (int32) and scores (fp32 bit
+patterns) must be identical, because both sides do the reference's fp32 additions in the
+reference's order and max is exact.  Calls go through the C ABI (i6fbw_viterbi) and through the
+Python interface that mirrors i6_native_ops.fast_viterbi."""
+import numpy as np
+import pytest
+import torch
+
+from i6_native_ops_amd import cabi
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import random_fsa
+from tests.test_oracle_viterbi import viterbi_fixture
+
+pytestmark = pytest.mark.gpu
+
+
+def run_cabi_viterbi(am, edges, weights, start_end, seq_lens, n_states, check=True):
+    dev = torch.device("cuda:0")
+    T, B, F = am.shape
+    E = int(edges.shape[1])
+    d_am = torch.from_numpy(np.ascontiguousarray(am)).to(dev)
+    d_edges = torch.from_numpy(np.ascontiguousarray(edges)).to(dev)
+    d_w = torch.from_numpy(np.ascontiguousarray(weights)).to(dev)
+    d_se = torch.from_numpy(np.ascontiguousarray(start_end)).to(dev)
+    d_len = torch.from_numpy(np.ascontiguousarray(seq_lens)).to(dev)
+    align = torch.full((T, B), -7, dtype=torch.int32, device=dev)
+    scores = torch.full((B,), 123.0, dtype=torch.float32, device=dev)
+    nbytes = cabi.workspace_size(T, B, F, E, n_states)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    print(f"viterbi T={T} B={B} F={F} E={E} S={n_states}", flush=True)
+    cabi.viterbi(d_am.data_ptr(), d_am.stride(0), d_am.stride(1), d_edges.data_ptr(), d_edges.stride(0) if E else 0,
+                 d_w.data_ptr(), d_se.data_ptr(), d_se.stride(0), d_len.data_ptr(), T, B, F, E, int(n_states),
+                 align.data_ptr(), align.stride(0), align.stride(1), scores.data_ptr(), ws.data_ptr(), nbytes, stream)
+    code, seq = cabi.read_status(ws.data_ptr(), B, stream)
+    if check and code != 0:
+        raise cabi.FbwError(code, seq)
+    torch.cuda.synchronize()
+    return align.cpu().numpy(), scores.cpu().numpy(), code
+
+
+def assert_identical(got, want):
+    (ga, gs), (wa, ws) = got, want
+    np.testing.assert_array_equal(ga, wa)
+    np.testing.assert_array_equal(gs.view(np.uint32), ws.view(np.uint32))
+
+
+def test_reference_vector(oracle):
+    args = viterbi_fixture()
+    align, scores, _ = run_cabi_viterbi(*args)
+    assert align[:, 0].tolist() == [0, 0, 1, 1, 1]            # test/fast_viterbi.py:39
+    assert_identical((align, scores), oracle.viterbi_oracle(*args))
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_automata(oracle, seed):
+    rng = np.random.default_rng(8100 + seed)
+    am, edges, weights, start_end, seq_lens, n_states = random_fsa(rng, B=int(rng.integers(1, 5)), F=int(rng.integers(2, 40)),
+                                                                   T=int(rng.integers(1, 12)))
+    am = -am
+    if seed % 4 == 0:
+        seq_lens[0] = 0
+    if seed % 5 == 0:
+        # coarse values make exact ties between candidates common
+        am = np.round(am)
+        weights = np.round(weights * 2) / 2
+    got = run_cabi_viterbi(am, edges, weights, start_end, seq_lens, n_states)[:2]
+    assert_identical(got, oracle.viterbi_oracle(am, edges, weights, start_end, seq_lens, n_states))
+
+
+def test_hand_worked_cases(oracle):
+    """The tie, no-path and zero-length cases that pin the oracle, on the GPU."""
+    am = np.zeros((2, 1, 6), dtype=np.float32)
+    diamond = np.array([[0, 1, 1, 0], [0, 2, 2, 0], [2, 3, 4, 0], [1, 3, 5, 0]], dtype=np.int32).T.copy()
+    a, s, _ = run_cabi_viterbi(am, diamond, np.zeros(4, np.float32), np.array([[0], [3]], np.int32), np.array([2], np.int32), 4)
+    assert a[:, 0].tolist() == [2, 4] and s[0] == 0.0
+    one = np.array([[0, 1, 5, 0]], dtype=np.int32).T.copy()
+    a, s, _ = run_cabi_viterbi(am, one, np.zeros(1, np.float32), np.array([[0], [1]], np.int32), np.array([2], np.int32), 2)
+    assert a[:, 0].tolist() == [5, 0] and s[0] == -np.inf
+    two = np.array([[0, 0, 1, 0], [1, 2, 2, 1]], dtype=np.int32).T.copy()
+    am2 = np.zeros((3, 2, 4), dtype=np.float32)
+    a, s, _ = run_cabi_viterbi(am2, two, np.zeros(2, np.float32), np.array([[0, 1], [0, 2]], np.int32), np.array([0, 0], np.int32), 3)
+    assert (a == 0).all() and s.tolist() == [0.0, -np.inf]
+
+
+@pytest.mark.parametrize("name", ["tiny", "monophone", "ctc"])
+@pytest.mark.parametrize("shuffle", [False, True])
+def test_workloads(oracle, name, shuffle):
+    wl = make_workload(name, shuffle_edges=shuffle)
+    am, w = -wl.am_scores, -wl.weights
+    got = run_cabi_viterbi(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states)[:2]
+    want = oracle.viterbi_oracle(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states)
+    assert np.isfinite(want[1]).all()
+    assert_identical(got, want)
+
+
+@pytest.mark.parametrize("kind", ["cart_small", "large_states", "large_emissions"])
+def test_size_classes(oracle, kind):
+    """Chains that take the one-state-per-thread path, the strided path (more than 512 states) and the
+    looped loader (more than 512 distinct emissions)."""
+    if kind == "cart_small":
+        wl = make_workload("cart", T=300, B=4, F=12001, n_labels=(60, 90))
+    elif kind == "large_states":
+        wl = make_workload("cart", T=900, B=2, F=300, n_labels=(250, 280))
+    else:
+        wl = make_workload("cart", T=900, B=2, F=12001, n_labels=(250, 280))
+    wl.seq_lens[:] = wl.T          # long enough for the longest chain
+    am, w = -wl.am_scores, -wl.weights
+    got = run_cabi_viterbi(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states)[:2]
+    assert_identical(got, oracle.viterbi_oracle(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states))
+
+
+def test_device_status():
+    """A state with more than eight incoming edges is reported, its sequence gets score NaN and zeros."""
+    n = 10
+    edges = np.array([[s, n, s % 3, 0] for s in range(n)] + [[0, s, 1, 0] for s in range(1, n)], dtype=np.int32).T.copy()
+    am = np.zeros((2, 1, 4), dtype=np.float32)
+    a, s, code = run_cabi_viterbi(am, edges, np.zeros(edges.shape[1], np.float32), np.array([[0], [n]], np.int32),
+                                  np.array([2], np.int32), n + 1, check=False)
+    assert code == -12 and np.isnan(s[0]) and (a == 0).all()
+
+
+def test_python_interface(oracle):
+    """align_viterbi(log_probs (B,T,F), fsa, seq_lens) -> ((B,T) int32, (B,)) as in
+    i6_native_ops/fast_viterbi/__init__.py:23-47, and core.fast_viterbi on (T,B,F)."""
+    from i6_native_ops_amd.fast_viterbi import align_viterbi, core
+    am, edges, weights, start_end, seq_lens, n = viterbi_fixture()
+    dev = "cuda:0"
+    log_probs = torch.from_numpy(am).to(dev).transpose(0, 1).contiguous()       # (B, T, F)
+    fsa = (n, torch.from_numpy(edges).to(dev), torch.from_numpy(weights).to(dev), torch.from_numpy(start_end).to(dev))
+    output, scores = align_viterbi(log_probs, fsa, torch.from_numpy(seq_lens).to(dev))
+    assert output.shape == (1, 5) and output.dtype == torch.int32 and scores.shape == (1,)
+    assert list(output[0].cpu()) == [0, 0, 1, 1, 1]
+    want = oracle.viterbi_oracle(am, edges, weights, start_end, seq_lens, n)
+    assert float(scores[0]) == float(want[1][0])
+
+    wl = make_workload("monophone")
+    lp = torch.from_numpy(-wl.am_scores).to(dev).transpose(0, 1).contiguous()
+    fsa = (wl.n_states, torch.from_numpy(wl.edges).to(dev), torch.from_numpy(-wl.weights).to(dev),
+           torch.from_numpy(wl.start_end_states).to(dev))
+    lens = torch.from_numpy(wl.seq_lens).to(dev)
+    out_bt, sc = align_viterbi(lp, fsa, lens)
+    out_tb, sc2 = core.fast_viterbi(lp.transpose(0, 1).contiguous(), fsa[1], fsa[2], fsa[3], lens, wl.n_states)
+    want = oracle.viterbi_oracle(-wl.am_scores, wl.edges, -wl.weights, wl.start_end_states, wl.seq_lens, wl.n_states)
+    np.testing.assert_array_equal(out_bt.cpu().numpy(), want[0].T)
+    np.testing.assert_array_equal(out_tb.cpu().numpy(), want[0])
+    np.testing.assert_array_equal(sc.cpu().numpy(), want[1])
+    np.testing.assert_array_equal(sc2.cpu().numpy(), want[1])
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        core.fast_viterbi(lp.cpu(), fsa[1], fsa[2], fsa[3], lens, wl.n_states)
