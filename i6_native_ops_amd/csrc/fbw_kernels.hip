@@ -368,7 +368,9 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     if (s_bad || st_state >= (unsigned)a.n_states || en_state >= (unsigned)a.n_states) err = I6FBW_ERR_BAD_INDEX;
     else if (n_edges > EB_MAX) err = I6FBW_ERR_SEQ_TOO_MANY_EDGES;
     const unsigned sl = (unsigned)a.seq_lens[b];
-    const int L = (sl >= 1u && sl <= (unsigned)a.T) ? (int)sl : 0;
+    // full sum: a length outside [1, T] leaves the sequence without probability mass; best path:
+    // lengths beyond T are read as T
+    const int L = a.best_path ? ((int)sl < 0 ? 0 : min((int)sl, a.T)) : ((sl >= 1u && sl <= (unsigned)a.T) ? (int)sl : 0);
     long long S = (long long)smax - smin + 1;
     if (!err && n_edges > 0 && S > 2LL * n_edges + 2) err = I6FBW_ERR_SEQ_SPARSE_STATES;
     if (n_edges == 0) S = 1;
@@ -562,7 +564,8 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
         }
         __syncthreads();
         int2* tb = a.tband + goff;
-        for (int d = tid; d < DP; d += 1024) tb[d] = make_int2(s_tlo[d], s_thi[d]);
+        // (the best-path search reads every frame: values outside the band would have to be -inf there)
+        for (int d = tid; d < DP; d += 1024) tb[d] = a.best_path ? make_int2(0, 1 << 30) : make_int2(s_tlo[d], s_thi[d]);
     }
 }
 

@@ -94,16 +94,18 @@ def test_workloads(oracle, name, shuffle):
     assert_identical(got, want)
 
 
-@pytest.mark.parametrize("kind", ["cart_small", "large_states", "large_emissions"])
+@pytest.mark.parametrize("kind", ["cart_small", "large_states", "large_emissions", "huge_states"])
 def test_size_classes(oracle, kind):
-    """Chains that take the one-state-per-thread path, the strided path (more than 512 states) and the
-    looped loader (more than 512 distinct emissions)."""
+    """Chains that take the one-state-per-thread path, the four-states-per-thread path (more than 512
+    states or distinct emissions) and the table-in-memory path (more than 2048 states)."""
     if kind == "cart_small":
         wl = make_workload("cart", T=300, B=4, F=12001, n_labels=(60, 90))
     elif kind == "large_states":
         wl = make_workload("cart", T=900, B=2, F=300, n_labels=(250, 280))
-    else:
+    elif kind == "large_emissions":
         wl = make_workload("cart", T=900, B=2, F=12001, n_labels=(250, 280))
+    else:
+        wl = make_workload("cart", T=2200, B=1, F=300, n_labels=(700, 710))
     wl.seq_lens[:] = wl.T          # long enough for the longest chain
     am, w = -wl.am_scores, -wl.weights
     got = run_cabi_viterbi(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states)[:2]
