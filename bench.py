@@ -33,6 +33,7 @@ def main():
     ap.add_argument("--workload", default="cart", help="tiny | monophone | cart | ctc | longform")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-wrapper", action="store_true", help="skip the wrapper-level (fbw_loss + backward) timing")
+    ap.add_argument("--no-best-path", action="store_true", help="skip the best-path (Viterbi) timing")
     ap.add_argument("--out-mode", type=int, default=1, help="0: -log posterior with +inf holes, 1: posterior")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise copy kernel over 1 GiB (3 times) so that a rocprofv3 --pmc run of "
@@ -167,6 +168,35 @@ def main():
             del lp
         result["config"]["wrapper_level"] = wl
         del base
+
+    # best path on the same automata (informational): i6fbw_viterbi maximises, so it gets -am and -weights
+    if not args.no_best_path:
+        vam = am.neg()
+        vw = weights.neg()
+        align = torch.empty((W.T, W.B), dtype=torch.int32, device=dev)
+        scores = torch.empty((W.B,), dtype=torch.float32, device=dev)
+
+        def vstep():
+            cabi.viterbi(vam.data_ptr(), vam.stride(0), vam.stride(1), edges.data_ptr(), edges.stride(0), vw.data_ptr(),
+                         start_end.data_ptr(), start_end.stride(0), seq_lens.data_ptr(), W.T, W.B, W.F, W.E, W.n_states,
+                         align.data_ptr(), align.stride(0), align.stride(1), scores.data_ptr(), ws.data_ptr(), ws_bytes,
+                         stream)
+        for _ in range(5):
+            vstep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            vstep()
+        torch.cuda.synchronize()
+        bp = {"ms_per_call": round((time.perf_counter() - t0) / 20 * 1e3, 4)}
+        if not args.no_cpu_baseline:
+            from oracle import fbw_oracle
+            t0 = time.perf_counter()
+            fbw_oracle.viterbi_oracle(-W.am_scores, W.edges, -W.weights, W.start_end_states, W.seq_lens, W.n_states)
+            bp["cpu_port_ms_per_call"] = round((time.perf_counter() - t0) * 1e3, 2)
+            bp["cpu_port_cores"] = 1
+        result["config"]["best_path"] = bp
+        del vam, vw
 
     if not args.no_cpu_baseline:
         from oracle import fbw_oracle
