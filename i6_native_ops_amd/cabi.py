@@ -18,7 +18,7 @@ STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
-           "i6fbw_set_overlap", "i6fbw_viterbi",
+           "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment", "i6fbw_set_band",
            "i6fbw_profile_enable", "i6fbw_profile_read")
 
 _lib = None
@@ -46,6 +46,14 @@ def load():
                                       c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
                                       c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
         lib.i6fbw_viterbi.restype = c.c_int
+        lib.i6fbw_dump_output.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_float,
+                                          c.c_uint, c.c_char_p, c.c_void_p]
+        lib.i6fbw_dump_output.restype = c.c_int
+        lib.i6fbw_dump_alignment.argtypes = [c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_void_p, c.c_int64, c.c_float,
+                                             c.c_uint, c.c_char_p, c.c_void_p]
+        lib.i6fbw_dump_alignment.restype = c.c_int
+        lib.i6fbw_set_band.argtypes = [c.c_int]
+        lib.i6fbw_set_band.restype = None
         lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
         lib.i6fbw_read_status.restype = c.c_int
         lib.i6fbw_strerror.argtypes = [c.c_int]
@@ -118,6 +126,25 @@ def read_status(ws_ptr, B, stream=0):
 def set_overlap(mode: int) -> None:
     """-1: by problem size, 0: single stream, 1: overlapped stages."""
     load().i6fbw_set_overlap(int(mode))
+
+
+def set_band(on: bool) -> None:
+    """False: gather every (frame, emission) score, needed before an alignment dump."""
+    load().i6fbw_set_band(1 if on else 0)
+
+
+def dump_alignment(ws_ptr, T, B, E, start_end_ptr, se_row_stride, pruning, batch_idx, directory, stream=0) -> None:
+    rc = load().i6fbw_dump_alignment(ws_ptr, T, B, E, start_end_ptr, se_row_stride, pruning, batch_idx,
+                                     os.fsencode(directory), stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def dump_output(out_ptr, out_stride_t, out_stride_b, seq_lens_ptr, T, B, F, pruning, batch_idx, directory, stream=0) -> None:
+    rc = load().i6fbw_dump_output(out_ptr, out_stride_t, out_stride_b, seq_lens_ptr, T, B, F, pruning, batch_idx,
+                                  os.fsencode(directory), stream)
+    if rc != 0:
+        raise FbwError(rc)
 
 
 def profile_enable(on: bool) -> None:

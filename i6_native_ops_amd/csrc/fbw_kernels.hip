@@ -24,7 +24,11 @@
 #include <string.h>
 
 #include <algorithm>
+#include <cmath>
+#include <cstdio>
 #include <mutex>
+#include <string>
+#include <vector>
 
 #include "../../include/i6fbw.h"
 
@@ -225,6 +229,7 @@ struct PrepArgs {
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
+    int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
@@ -565,7 +570,7 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
         __syncthreads();
         int2* tb = a.tband + goff;
         // (the best-path search reads every frame: values outside the band would have to be -inf there)
-        for (int d = tid; d < DP; d += 1024) tb[d] = a.best_path ? make_int2(0, 1 << 30) : make_int2(s_tlo[d], s_thi[d]);
+        for (int d = tid; d < DP; d += 1024) tb[d] = (a.best_path || a.no_band) ? make_int2(0, 1 << 30) : make_int2(s_tlo[d], s_thi[d]);
     }
 }
 
@@ -1402,6 +1407,7 @@ int g_groups = [] {
     const char* e = getenv("I6FBW_GROUPS");
     return e ? atoi(e) : 0;
 }();
+int g_no_band = 0;      // see i6fbw_set_band
 int g_overlap_mode = [] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
@@ -1468,7 +1474,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
-    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0;
+    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = g_no_band;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
@@ -1610,6 +1616,88 @@ void i6fbw_set_overlap(int mode) {
 int i6fbw_debug_trace(void* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * n); }
 int i6fbw_debug_trace_set(const void* host, int n) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), host, sizeof(unsigned long long) * n); }
 #endif
+
+void i6fbw_set_band(int on) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_no_band = on ? 0 : 1;
+}
+
+// Text dumps of fbw_op.cu:155-224.  Host code: device-to-host copies and file output.
+int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32_t* start_end, int64_t se_row_stride,
+                         float pruning, unsigned batch_idx, const char* directory, void* stream) {
+    if (!workspace || !start_end || !directory || T <= 0 || B <= 0 || E < 0) return I6FBW_ERR_INVALID_ARGUMENT;
+    const Layout l = make_layout(T, B, E);
+    std::vector<SeqMeta> meta(B);
+    std::vector<int32_t> se(2 * (size_t)B);
+    hipStream_t s = (hipStream_t)stream;
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipMemcpy(meta.data(), (const char*)workspace + l.meta, sizeof(SeqMeta) * B, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(se.data(), start_end, sizeof(int32_t) * B, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(se.data() + B, start_end + se_row_stride, sizeof(int32_t) * B, hipMemcpyDeviceToHost));
+    std::vector<float> rows;
+    for (int b = 0; b < B; b++) {
+        const std::string name = std::string(directory) + "/alignment.dump." + std::to_string(batch_idx) + "." + std::to_string(b);
+        FILE* f = fopen(name.c_str(), "w");
+        if (!f) return I6FBW_ERR_INVALID_ARGUMENT;
+        const SeqMeta& m = meta[b];
+        const bool ok = !(m.err || m.errA || m.errB);
+        const long long first = se[b], last = se[B + b];           // the reference walks the ids start..end
+        // frame 0 is written even for an empty sequence (fbw_op.cu:177); it holds the start state only
+        const int frames = !ok ? 0 : (m.L > 0 && m.n_edges > 0 ? m.L : 1);
+        const bool have_rows = ok && m.L > 0 && m.n_edges > 0;
+        if (have_rows) {
+            rows.resize((size_t)m.L * m.SP);
+            const float* src = (const float*)((const char*)workspace + l.alpha) + (size_t)T * state_off(m.edge_begin, b);
+            if (hipMemcpy(rows.data(), src, sizeof(float) * rows.size(), hipMemcpyDeviceToHost) != hipSuccess) { fclose(f); return I6FBW_ERR_LAUNCH; }
+        }
+        for (int t = 0; t < frames; t++) {
+            // value of state id s in natural-log units (rows are stored in units of log 2, relative
+            // to an offset that cancels in the normalisation)
+            auto value = [&](long long sid) -> float {
+                const long long loc = sid - m.state_min;
+                if (!have_rows) return sid == first ? 0.f : INFINITY;
+                if (loc < 0 || loc >= m.S) return INFINITY;
+                return rows[(size_t)t * m.SP + loc] * LN2;
+            };
+            float sum = INFINITY;
+            for (long long sid = first; sid <= last; sid++) {
+                const float val = value(sid);
+                const float diff = val - sum;
+                if (!std::isnan(diff)) sum = -log1pf(expf(-fabsf(diff))) + fminf(sum, val);
+            }
+            for (long long sid = first; sid <= last; sid++) {
+                const float val = value(sid) - sum;
+                if (val <= pruning) fprintf(f, "%d %lld %g\n", t, sid - first, val);
+            }
+        }
+        fclose(f);
+    }
+    return I6FBW_OK;
+}
+
+int i6fbw_dump_output(const float* out, int64_t out_stride_t, int64_t out_stride_b, const int32_t* seq_lens, int T, int B,
+                      int F, float pruning, unsigned batch_idx, const char* directory, void* stream) {
+    if (!out || !seq_lens || !directory || T <= 0 || B <= 0 || F <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    HIP_TRY(hipStreamSynchronize(s));
+    std::vector<int32_t> lens(B);
+    HIP_TRY(hipMemcpy(lens.data(), seq_lens, sizeof(int32_t) * B, hipMemcpyDeviceToHost));
+    std::vector<float> row(F);
+    for (int b = 0; b < B; b++) {
+        const std::string name = std::string(directory) + "/target.dump." + std::to_string(batch_idx) + "." + std::to_string(b);
+        FILE* f = fopen(name.c_str(), "w");
+        if (!f) return I6FBW_ERR_INVALID_ARGUMENT;
+        for (int t = 0; t < T; t++) {
+            if (t > 0 && (unsigned)t >= (unsigned)lens[b]) break;
+            if (hipMemcpy(row.data(), out + (int64_t)t * out_stride_t + (int64_t)b * out_stride_b, sizeof(float) * F,
+                          hipMemcpyDeviceToHost) != hipSuccess) { fclose(f); return I6FBW_ERR_LAUNCH; }
+            for (int e = 0; e < F; e++)
+                if (row[e] <= pruning) fprintf(f, "%d %d %g\n", t, e, row[e]);
+        }
+        fclose(f);
+    }
+    return I6FBW_OK;
+}
 
 const char* i6fbw_last_hip_error(void) { return g_last_hip_error == hipSuccess ? "" : hipGetErrorString(g_last_hip_error); }
 

@@ -44,7 +44,8 @@ static bool status_check_enabled() {
 // fused == true:  am_scores is log_probs (B, T, F) with unit innermost stride; out is (B, T, F).
 static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
                                       torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
-                                      int out_mode, bool fused = false) {
+                                      int out_mode, bool fused = false, const DebugOptions* dump = nullptr,
+                                      unsigned batch_idx = 0u) {
     if (fused) {
         CHECK_CUDA(am_scores);
         CHECK_TYPE(am_scores, torch::kFloat32);
@@ -80,12 +81,17 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc));
     torch::Tensor workspace = torch::empty({(int64_t)ws_bytes}, opts.dtype(torch::kUInt8));
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    // the alignment dump needs the forward scores of every state, also of those that cannot reach
+    // the end state any more
+    const bool all_scores = dump && dump->dump_alignment;
+    if (all_scores) i6fbw_set_band(0);
     rc = i6fbw_run_strided(am_scores.data_ptr<float>(), am_scores.stride(dt), am_scores.stride(db), fused ? 1 : 0,
                            edges.data_ptr<int32_t>(), edges.stride(0), weights.data_ptr<float>(),
                            start_end_states.data_ptr<int32_t>(), start_end_states.stride(0),
                            seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode, out.data_ptr<float>(),
                            out.stride(dt), out.stride(db), sum_output.data_ptr<float>(), workspace.data_ptr(), ws_bytes,
                            (void*)stream);
+    if (all_scores) i6fbw_set_band(1);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
     if (status_check_enabled()) {
         int code = 0, seq = -1;
@@ -93,14 +99,31 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
         TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
         TORCH_CHECK(code == I6FBW_OK, "NativeOp: fbw: sequence ", seq, ": ", i6fbw_strerror(code));
     }
+    if (dump && dump->dump_alignment) {
+        // as fbw_op.cu:361-364
+        rc = i6fbw_dump_alignment(workspace.data_ptr(), T, B, E, start_end_states.data_ptr<int32_t>(),
+                                  start_end_states.stride(0), dump->pruning, batch_idx, ".", (void*)stream);
+        TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: alignment dump: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
+    }
+    if (dump && dump->dump_output) {
+        // as fbw_op.cu:379-381
+        rc = i6fbw_dump_output(out.data_ptr<float>(), out.stride(dt), out.stride(db), seq_lens.data_ptr<int32_t>(), T, B, F,
+                               dump->pruning, batch_idx, ".", (void*)stream);
+        TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: output dump: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
+    }
     return {out, sum_output};
 }
 
 std::vector<torch::Tensor> fbw(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,
                                torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
                                DebugOptions debug_options = DebugOptions()) {
-    (void)debug_options;
-    return run(am_scores, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_NEG_LOG);
+    // calls are numbered as in the reference (fbw_op.cu:246,390); every dump_every-th one is dumped
+    static unsigned batch_idx = 0u;
+    const unsigned idx = batch_idx++;
+    const bool dump_now = (debug_options.dump_alignment || debug_options.dump_output) && debug_options.dump_every > 0u &&
+                          idx % debug_options.dump_every == 0u;
+    return run(am_scores, edges, weights, start_end_states, seq_lens, num_states, I6FBW_OUT_NEG_LOG, false,
+               dump_now ? &debug_options : nullptr, idx);
 }
 
 std::vector<torch::Tensor> fbw_posterior(torch::Tensor& am_scores, torch::Tensor& edges, torch::Tensor& weights,

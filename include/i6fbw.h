@@ -153,6 +153,31 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
  */
 void i6fbw_set_overlap(int mode);
 
+/*
+ * Debug dumps of the reference (fbw_op.cu:155-224, switched by DebugOptions, DebugOptions.h:4-9).
+ * Host-side helpers: they synchronise `stream`, copy to the host and write one text file per
+ * sequence into `directory` (the reference writes into the working directory).
+ *
+ * i6fbw_dump_output: file target.dump.<batch_idx>.<seq>, a line "t e value" for every element of
+ * out[t, seq, :] (as written with I6FBW_OUT_NEG_LOG) that is <= pruning, for t < seq_lens[seq]
+ * (frame 0 always), as write_output_to_file (fbw_op.cu:199-224).
+ *
+ * i6fbw_dump_alignment: file alignment.dump.<batch_idx>.<seq>, a line "t (state - start) value"
+ * for the states start..end of the sequence, where value = forward score of the state before
+ * frame t minus the log-sum over those states, if <= pruning, as write_alignment_to_file
+ * (fbw_op.cu:155-197).  It reads the forward rows of the last i6fbw_run on `workspace`; call
+ * i6fbw_set_band(0) before that run, otherwise states that cannot reach the end state in the
+ * remaining frames are missing (their scores are never computed), and i6fbw_set_band(1) after it.
+ * Sequences whose length is outside [1, T] have no forward rows: frame 0 alone is written.
+ */
+int i6fbw_dump_output(const float* out, int64_t out_stride_t, int64_t out_stride_b, const int32_t* seq_lens,
+                      int T, int B, int F, float pruning, unsigned batch_idx, const char* directory, void* stream);
+int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32_t* start_end, int64_t se_row_stride,
+                         float pruning, unsigned batch_idx, const char* directory, void* stream);
+/* 1 (default): scores outside the frames in which an emission can carry mass are not gathered;
+ * 0: all are (slower, same outputs; needed for i6fbw_dump_alignment).  Process-wide. */
+void i6fbw_set_band(int on);
+
 /* Text for a status code. */
 const char* i6fbw_strerror(int code);
 
