@@ -63,10 +63,15 @@ constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of t
 constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup
 constexpr int REC_LOADERS = 1;        // loader waves beside them
 constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
+// Two recursion workgroups share a compute unit only if a workgroup has at most eight waves
+// (measured: nine-wave workgroups with this much LDS are placed one per unit): the instance for
+// batches with more workgroups than compute units runs 448 compute threads beside the loader wave.
+constexpr int REC_THREADS_DENSE = 448;
+constexpr int REC_BLOCK_DENSE = REC_THREADS_DENSE + 64 * REC_LOADERS;
 constexpr unsigned NO_STATE = 0xFFFFu;
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
 constexpr int SYNC_HDR = 16;          // ints before the progress counters in the hand-off area:
-                                      // [0] abort flag, [1] recursion workgroups placed so far
+                                      // [0] abort flag, [1] recursion workgroups placed so far, [3] preparation workgroups finished
 constexpr int PUBLISH = 32;           // recursion steps between progress publications
 constexpr int SPIN_LIMIT = 1 << 20;   // polls before a waiting wave gives up
 // Scores are kept in units of log 2 inside the workspace (exp2/log2 are single instructions).
@@ -136,11 +141,11 @@ __device__ unsigned long long g_trace[4096];   // debug builds only: in-kernel t
 __device__ inline int seq_error(const SeqMeta& m) { return m.err ? m.err : (m.errA ? m.errA : m.errB); }
 
 // Recursion class of a sequence: 0 nothing to do, 1..3 by size, -1 error.
-__device__ inline int rec_class(const SeqMeta& m) {
+__device__ inline int rec_class(const SeqMeta& m, const int threads = REC_THREADS) {
     if (seq_error(m)) return -1;
     if (m.L == 0 || m.n_edges == 0) return 0;
-    if (m.SP <= REC_THREADS && m.DP <= 512) return 1;
-    if (m.SP <= 4 * REC_THREADS && m.DP <= 2048) return 2;
+    if (m.SP <= threads && m.DP <= 512) return 1;
+    if (m.SP <= 4 * threads && m.DP <= 2048) return 2;
     return 3;
 }
 
@@ -236,8 +241,10 @@ struct PrepArgs {
 // sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never
 // decrease.  Where the index steps up, the first edge of every sequence in between is recorded:
 // seqbegin[q] = first edge with sequence index >= q (valid if the whole list turns out sorted).
-__global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int E, int B, int* sortflag, int* seqbegin) {
+// As the first kernel of a call it also clears the header of the hand-off area.
+__global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int E, int B, int* sortflag, int* seqbegin, int* sync) {
     __shared__ int bad;
+    if (blockIdx.x == 0 && threadIdx.x < SYNC_HDR) sync[threadIdx.x] = 0;
     if (threadIdx.x == 0) bad = 0;
     __syncthreads();
     const int base = blockIdx.x * SCAN_BLOCK;
@@ -305,7 +312,7 @@ __device__ inline int min_steps(int from, int to, int dmax, int dmin) {
 // state (beta), role 2 by emission slot (combine) and writes the shared part of the meta record.
 // For edge lists grouped by sequence (the usual case) the scan kernel has recorded where each
 // sequence starts; any other order is handled by a stable scan over the whole list.
-__global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
+__device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     __shared__ unsigned keys[EB_MAX];
     __shared__ unsigned bitmap[F_BITMAP_MAX / 32];
     __shared__ int wordpfx[F_BITMAP_MAX / 32];
@@ -417,7 +424,6 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     if (role == 2) {
         // hand-off area of this sequence: progress counters and gather flags start at zero
         const int nstrip = (a.T + TG - 1) / TG;
-        if (b == 0 && tid < SYNC_HDR) a.sync[tid] = 0;
         if (tid < 2) a.sync[SYNC_HDR + 2 * b + tid] = 0;
         int* gf = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * nstrip;
         for (int i = tid; i < nstrip; i += 1024) gf[i] = 0;
@@ -574,6 +580,14 @@ __global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
     }
 }
 
+__global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
+    prepare_sequence(a);      // every exit from it is taken by the whole workgroup
+    // The recursion kernel of the overlapped schedule is already on the machine and waits for this
+    // count: write this workgroup's tables back from the L2 of its XCD before it is raised.
+    __syncthreads();
+    if (threadIdx.x == 0) { __threadfence(); atomicAdd(&a.sync[3], 1); }
+}
+
 // ---------------------------------------------------------------------------------------------
 // stage 2: gather  gtab[b][t][slot] = log2(e) * am[t, b, demis[b][slot]]  for t < L_b.
 // Strips of TG frames are handed out from both ends of a sequence towards its middle, the order in
@@ -638,6 +652,7 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
 // ---------------------------------------------------------------------------------------------
 struct RecArgs {
     int T, B;
+    int prep_wgs;     // workgroups of the preparation kernel
     const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab;
     float* alpha; float* beta; double* offA; double* offB;
     int* sync;
@@ -939,25 +954,38 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
 }
 
 // REC_THREADS compute threads plus one loader wave per workgroup; grid = 2B.
-// DENSE caps the register use (5 waves per SIMD) so that two workgroups fit on a compute unit;
-// the host picks it when the batch has more workgroups than the device has compute units.  The
-// rarely used large-automaton paths pay for the cap with spills, which is why small batches run
-// the uncapped instance.
+// DENSE is the instance of which two workgroups fit on a compute unit: eight waves, and at most 96
+// registers -- two workgroups are four waves per SIMD, and the rest of the register file is what
+// the gate, gather and combine waves need to get onto the unit at all.
+// The host picks it when the batch has more workgroups than the device has compute units.  The rarely used large-automaton paths pay for the cap with spills,
+// which is why small batches run the uncapped instance.
 template <bool SYNC, bool DENSE>
-__global__ __launch_bounds__(REC_BLOCK, DENSE ? 5 : 1) void fbw_recurse(RecArgs a) {
-    constexpr int T_ = REC_THREADS, NW = T_ / 64;
-    __shared__ float st[2][S_MAX + 16];
-    __shared__ __attribute__((aligned(16))) float amr[2][D_MAX];
-    __shared__ float wmin[NW];
+__device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) {
+    constexpr int T_ = DENSE ? REC_THREADS_DENSE : REC_THREADS;
+    // LDS of a workgroup (REC_LDS_FLOATS floats, 16-byte aligned): the emission rows first
+    float (*amr)[D_MAX] = (float (*)[D_MAX])lds;
+    float (*st)[S_MAX + 16] = (float (*)[S_MAX + 16])(lds + 2 * D_MAX);
+    float* wmin = lds + 2 * D_MAX + 2 * (S_MAX + 16);
+    int* go_flag = (int*)(wmin + 8);
 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
     // gather or combine waves
     __builtin_amdgcn_s_setprio(3);
-    // every workgroup reports that it has been placed (see fbw_gate)
-    if (SYNC && threadIdx.x == 0) atomicAdd(&a.sync[1], 1);
+    if (SYNC) {
+        // This kernel is started beside the preparation, so that its large workgroups are placed
+        // while the machine is still empty: report the placement (see fbw_gate), wait until all
+        // preparation workgroups have counted themselves, then drop stale cache lines.
+        if (threadIdx.x == 0) {
+            atomicAdd(&a.sync[1], 1);
+            *go_flag = spin_until_ge(a.sync + 3, a.prep_wgs, a.sync) ? 1 : 0;
+        }
+        __syncthreads();
+        if (!*go_flag) return;
+        __threadfence();
+    }
     const int b = blockIdx.x >> 1, dir = blockIdx.x & 1;
     const SeqMeta m = a.meta[b];
-    const int cls = rec_class(m);
+    const int cls = rec_class(m, T_);
     if (cls <= 0) return;
     const bool loader = threadIdx.x >= T_;
     const int K = dir ? m.Kout : m.Kin;
@@ -980,6 +1008,21 @@ __global__ __launch_bounds__(REC_BLOCK, DENSE ? 5 : 1) void fbw_recurse(RecArgs 
         if (loader) recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
         else recurse_compute_generic<SYNC, T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, S_MAX);
     }
+}
+
+constexpr int REC_LDS_FLOATS = 2 * D_MAX + 2 * (S_MAX + 16) + 8 + 8;
+template <bool SYNC>
+__global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS];
+    recurse_workgroup<SYNC, false>(a, lds);
+}
+// The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS floats): with the
+// size known at compile time the compiler sees that at most two workgroups fit on a unit anyway
+// and ignores the register cap, and two workgroups then fill the register file.
+template <bool SYNC>
+__global__ __launch_bounds__(REC_BLOCK_DENSE, 5) void fbw_recurse_dense(RecArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
+    recurse_workgroup<SYNC, true>(a, dyn_lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1274,7 +1317,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     }
 }
 
-// One-time check that two library streams really run at the same time (see pipeline_init).
+// Check that two streams really run at the same time (see runs_beside).
 __device__ int g_selftest[4];
 __global__ void fbw_selftest_wait() {
     if (threadIdx.x == 0) {
@@ -1323,16 +1366,18 @@ thread_local hipError_t g_last_hip_error = hipSuccess;
         if (e_ != hipSuccess) { g_last_hip_error = e_; return I6FBW_ERR_LAUNCH; } \
     } while (0)
 
-// Library-owned streams and events of one device.  A large call keeps the edge preparation and
-// the dense write (the first and the last kernel) on the caller's stream and runs the padding
-// fill, the gather and the recursion beside them on three streams of its own; the kernels that run
-// at the same time feed each other through flags in memory.
+// Library-owned streams and events of one device.  A large call keeps the edge preparation, the
+// gather and the dense write on the caller's stream and runs the padding fill and the recursion
+// beside them on two streams of its own; the kernels that run at the same time feed each other
+// through flags in memory.
 struct Pipeline {
     bool ready = false;
-    hipStream_t sP = nullptr, sG = nullptr, sR = nullptr;
-    hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneG = nullptr, doneR = nullptr;
+    hipStream_t sP = nullptr, sR = nullptr;
+    hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneR = nullptr;
     int n_cu = 256;
-    bool concurrent = false;     // the recursion and gather streams were seen running at the same time
+    // caller streams that were checked against the recursion stream: do kernels on the two run at
+    // the same time?
+    std::vector<std::pair<hipStream_t, bool>> checked;
 };
 Pipeline g_pipe[MAX_DEVICES];
 std::mutex g_mutex;
@@ -1344,27 +1389,36 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipDeviceGetAttribute(&p.n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     // default priority on purpose
     HIP_TRY(hipStreamCreateWithFlags(&p.sP, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&p.sG, hipStreamNonBlocking));
     HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
-    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneG, &p.doneR})
+    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, 90 * 1024));
+        HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-    // The overlapped schedule enqueues the recursion before the gather it waits for (so that its
-    // workgroups are placed at once).  That only works if the two streams are served at the same
-    // time; check it once with a bounded handshake and fall back to the single-stream schedule if
-    // the waiter never sees the flag (e.g. both streams mapped to one hardware queue).
-    fbw_selftest_set<<<1, 64, 0, p.sG>>>(0);
-    HIP_TRY(hipStreamSynchronize(p.sG));
+    p.ready = true;
+    return I6FBW_OK;
+}
+
+// In the overlapped schedule the recursion kernel (library stream) waits in memory for kernels that
+// the caller's stream starts after it.  That only works if the two streams are served at the same
+// time; the first large call on a stream checks it with a bounded handshake between two one-wave
+// kernels (this synchronises the stream once), and the single-stream schedule is used if the waiter
+// never sees the flag (e.g. both streams mapped to one hardware queue, or a serialising profiler).
+int runs_beside(Pipeline& p, hipStream_t s, bool* yes) {
+    for (const auto& c : p.checked)
+        if (c.first == s) { *yes = c.second; return I6FBW_OK; }
+    fbw_selftest_set<<<1, 64, 0, s>>>(0);
+    HIP_TRY(hipStreamSynchronize(s));
     fbw_selftest_wait<<<1, 64, 0, p.sR>>>();
-    fbw_selftest_set<<<1, 64, 0, p.sG>>>(1);
+    fbw_selftest_set<<<1, 64, 0, s>>>(1);
     HIP_TRY(hipStreamSynchronize(p.sR));
-    HIP_TRY(hipStreamSynchronize(p.sG));
+    HIP_TRY(hipStreamSynchronize(s));
     int result[4] = {0, 0, 0, 0};
     HIP_TRY(hipMemcpyFromSymbol(result, HIP_SYMBOL(g_selftest), sizeof(result)));
-    p.concurrent = result[1] == 1;
-    p.ready = true;
+    *yes = result[1] == 1;
+    if (p.checked.size() >= 64) p.checked.clear();
+    p.checked.emplace_back(s, *yes);
     return I6FBW_OK;
 }
 
@@ -1461,8 +1515,15 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     int* sync = (int*)(ws + l.sync);
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
     const int forced = g_overlap_mode;
-    const bool overlap = P.concurrent && (forced >= 0 ? forced != 0 : (long long)T * B * F >= (1LL << 26));
-    hipStream_t sP = overlap ? P.sP : s, sG = overlap ? P.sG : s, sR = overlap ? P.sR : s;
+    // By default only where it pays: a large dense tensor, and a batch whose recursion workgroups
+    // leave wave slots free on every compute unit (with two of them on each unit the gather crawls:
+    // T=200, B=256, F=5001 takes 0.59 ms overlapped against 0.48 ms stage after stage).
+    bool overlap = forced >= 0 ? forced != 0 : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu);
+    // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
+    // unit): gather and dense write wait for their progress while occupying wave slots themselves.
+    if (2 * B > 2 * P.n_cu) overlap = false;
+    if (overlap) { int rc = runs_beside(P, s, &overlap); if (rc != I6FBW_OK) return rc; }
+    hipStream_t sP = overlap ? P.sP : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;
 
     // blocks of sequences for the hand-out order of gather and combine (see grouped_index)
@@ -1478,36 +1539,12 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
-    {
-        StageTimer tm(0, s);
-        if (E > 0) {
-            hipLaunchKernelGGL(fbw_scan_sorted, dim3((E + SCAN_BLOCK - 1) / SCAN_BLOCK), dim3(256), 0, s,
-                               edges + 3 * edge_row_stride, E, B, pa.sortflag, pa.seqbegin);
-            HIP_TRY(hipGetLastError());
-        }
-        if (overlap) HIP_TRY(hipEventRecord(P.start, s));      // releases the padding fill, see below
-        hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
-        HIP_TRY(hipGetLastError());
-    }
-    // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
-    // leaves the memory system idle.  The fill is released when the scan kernel is done, i.e. when
-    // the preparation's large workgroups are being placed, so that its many small workgroups
-    // cannot keep them off the machine.
-    if (overlap) HIP_TRY(hipStreamWaitEvent(sP, P.start, 0));
-    {
-        StageTimer tm(4, sP);
-        hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
-                           (long long)out_stride_b, sum_output);
-        HIP_TRY(hipGetLastError());
-    }
-    if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
-
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
     ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.per_group = per_group;
     RecArgs ra;
-    ra.T = T; ra.B = B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
+    ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
     ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.sync = sync;
     CombArgs ca;
@@ -1517,54 +1554,89 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync; ca.per_group = per_group;
     const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
+    {
+        // the scan also clears the header of the hand-off area, so it runs even without edges
+        StageTimer tm(0, s);
+        hipLaunchKernelGGL(fbw_scan_sorted, dim3(std::max(1, (E + SCAN_BLOCK - 1) / SCAN_BLOCK)), dim3(256), 0, s,
+                           edges + 3 * edge_row_stride, E, B, pa.sortflag, pa.seqbegin, sync);
+        HIP_TRY(hipGetLastError());
+    }
+    // Where the recursion kernel is started: beside the preparation if its 2B workgroups leave at
+    // least half of the compute units empty (the preparation's workgroups need most of a unit's
+    // LDS and could otherwise find no room while the recursion waits for them), else behind it.
+    const bool early = overlap && 2 * B <= P.n_cu / 2;
+    auto launch_recursion = [&]() -> int {
+        { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS, sR, ra);
+          else hipLaunchKernelGGL(fbw_recurse<true>, dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipEventRecord(P.doneR, sR));
+        return I6FBW_OK;
+    };
+    if (overlap) {
+        // The library streams are released when the scan is done, i.e. while the preparation's
+        // workgroups are being placed.  The recursion's 2B large workgroups need ten free wave
+        // slots on one compute unit each and find them while the machine is still almost empty;
+        // they wait in memory for the preparation to finish (fbw_prepare counts its workgroups),
+        // and their loader waves later for the gather's strip flags.
+        HIP_TRY(hipEventRecord(P.start, s));
+        HIP_TRY(hipStreamWaitEvent(sP, P.start, 0));
+        if (early) {
+            HIP_TRY(hipStreamWaitEvent(sR, P.start, 0));
+            int rc = launch_recursion(); if (rc != I6FBW_OK) return rc;
+        }
+    }
+    {
+        StageTimer tm(0, s);
+        hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
+        HIP_TRY(hipGetLastError());
+    }
+    if (overlap && !early) {
+        HIP_TRY(hipEventRecord(P.fork, s));
+        HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
+        int rc = launch_recursion(); if (rc != I6FBW_OK) return rc;
+    }
+    // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
+    // leaves the memory system idle.
+    {
+        StageTimer tm(4, sP);
+        hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
+                           (long long)out_stride_b, sum_output);
+        HIP_TRY(hipGetLastError());
+    }
+    if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
+
     if (!overlap) {
         { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL((fbw_recurse<false, true>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra);
-          else hipLaunchKernelGGL((fbw_recurse<false, false>), dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
+        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS, s, ra);
+          else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
         { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
         HIP_TRY(hipGetLastError());
         return I6FBW_OK;
     }
 
-    HIP_TRY(hipEventRecord(P.fork, s));
-    HIP_TRY(hipStreamWaitEvent(sG, P.fork, 0));
-    HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
-    // The recursion goes first so that its 2B workgroups are placed before the gather fills the
-    // machine; its loader waves wait for the gather's strip flags (pipeline_init has checked that
-    // the two streams run side by side).  Every other in-kernel wait is for a kernel enqueued earlier.
-    { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
-      else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
-    HIP_TRY(hipGetLastError());
-    HIP_TRY(hipEventRecord(P.doneR, sR));
-    // A recursion workgroup needs ten free wave slots on one compute unit at once; a running grid of
-    // small workgroups refills every slot it frees, so the gather is held back until all recursion
-    // workgroups have been placed.
-    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sG, sync, 2 * B);
+    // A running grid of small workgroups refills every wave slot it frees, so gather and dense
+    // write (which also wait for recursion progress while they occupy LDS and wave slots) are
+    // held back until every recursion workgroup is on the machine -- normally long since.
+    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
     HIP_TRY(hipGetLastError());
 #ifndef I6_GATHER_LDS
 #define I6_GATHER_LDS 0
 #endif
-    { StageTimer tm(1, sG); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), I6_GATHER_LDS, sG, ga); }
+    { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), I6_GATHER_LDS, s, ga); }
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipEventRecord(P.doneG, sG));
-    // The dense write is the last kernel on the caller's stream.  It starts when the gather is
-    // done (its workgroups would only take wave slots away from the gather before that: by then the
-    // two recursions are about to meet in the middle of the sequences, where the dense write
-    // begins) and the gate has seen every recursion workgroup on the machine; from then on each
-    // of its workgroups waits for the recursion progress it needs.
-    if (groups == 1) HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
+    // The dense write follows the gather on the same stream (its workgroups would only take wave
+    // slots away from the gather before that: by then the two recursions are about to meet in the
+    // middle of the sequences, where the dense write begins); each of its workgroups waits for the
+    // recursion progress it needs.
 #ifdef I6_TRACE
     if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
 #endif
-    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
-    HIP_TRY(hipGetLastError());
     { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
     HIP_TRY(hipGetLastError());
-    // join: all three finish well before the dense write does
+    // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
-    HIP_TRY(hipStreamWaitEvent(s, P.doneG, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     return I6FBW_OK;
 }

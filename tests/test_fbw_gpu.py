@@ -70,6 +70,9 @@ def test_random_automata_brute_force(oracle, seed):
     ("cart", dict(T=300, B=3, F=12001, shuffle_edges=True)),
     ("ctc", dict(T=40, B=8, F=50)),
     ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
+    ("ctc", dict(T=30, B=200, F=40)),          # 400 recursion workgroups: two per compute unit, started behind the preparation
+    ("ctc", dict(T=30, B=256, F=40)),          # exactly two recursion workgroups on every compute unit
+    ("ctc", dict(T=24, B=600, F=40)),          # more recursion workgroups than the device holds at once
     ("longform", dict(T=200, B=2, F=300)),
     ("longform", dict(T=1200, B=2, F=999, n_labels=(150, 200))),     # > 512 states: second size class
     ("longform", dict(T=4000, B=1, F=777, n_labels=(700, 800))),     # > 2048 states: third size class
