@@ -627,7 +627,7 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
 #pragma unroll
         for (int tt = 0; tt < TG; tt++) {
             v[tt] = INF_F;
-            if (tt < nt && t0 + tt >= band.x && t0 + tt <= band.y) v[tt] = am[(long long)(t0 + tt) * a.st_t + e];
+            if (tt < nt && t0 + tt >= band.x && t0 + tt <= band.y) v[tt] = __builtin_nontemporal_load(&am[(long long)(t0 + tt) * a.st_t + e]);   // read once: keep it out of the caches
         }
 #pragma unroll
         for (int tt = 0; tt < TG; tt++)
