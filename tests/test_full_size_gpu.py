@@ -1,0 +1,90 @@
+"""The configurations of the benchmark at their full sizes: size-independent properties of the
+result (every valid row of the posterior sums to 1, the loss is the same in every valid frame of a
+sequence and 0 after it, holes exactly where no edge of the sequence carries the emission, padding
+rows empty, result independent of the edge order) and, since the CPU oracle finishes them in
+seconds with a few threads, the full comparison too."""
+import numpy as np
+import pytest
+import torch
+
+from i6_native_ops_amd import cabi
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.gpu_util import DeviceProblem
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name", ["cart", "ctc", "longform"])
+def test_full_size(oracle, name):
+    W = make_workload(name)
+    print(f"full size {name}: T={W.T} B={W.B} F={W.F} E={W.E}", flush=True)
+    P = DeviceProblem(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    post, loss = P.run(cabi.OUT_PROB)
+    torch.cuda.synchronize()
+    lens = torch.from_numpy(W.seq_lens).to(post.device)
+    valid = torch.arange(W.T, device=post.device)[:, None] < lens[None, :]            # (T, B)
+
+    rowsum = post.sum(-1, dtype=torch.float64)
+    assert torch.all((rowsum[valid] - 1.0).abs() < 1e-4)                              # test/fbw.py:60-64
+    assert torch.all(rowsum[~valid] == 0)
+    assert torch.all(post >= 0) and torch.all(post <= 1.0 + 1e-5)
+    # loss: one value per sequence, repeated in its valid frames, 0 afterwards
+    first = loss[0][None, :].expand_as(loss)
+    assert torch.all(((loss - first).abs() <= 1e-5 * first.abs())[valid])
+    assert torch.all(loss[~valid] == 0)
+    # holes: posterior mass only on emissions that some edge of the sequence carries
+    allowed = torch.zeros((W.B, W.F), dtype=torch.bool, device=post.device)
+    allowed[torch.from_numpy(W.edges[3].astype(np.int64)).to(post.device),
+            torch.from_numpy(W.edges[2].astype(np.int64)).to(post.device)] = True
+    assert torch.all(post.amax(0)[~allowed] == 0)
+
+    # the oracle on the whole problem
+    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens,
+                                            W.n_states, threads=min(16, W.B))
+    np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
+    got = post.cpu().numpy()
+    worst = 0.0
+    for t0 in range(0, W.T, 100):                       # in slices: exp() of the whole tensor at once is 12 GB in float64
+        ref = np.exp(-want_out[t0:t0 + 100].astype(np.float64))
+        worst = max(worst, float(np.abs(got[t0:t0 + 100] - ref).max()))
+    assert worst <= 1e-4
+    del got, want_out
+
+    # same problem with the edge list shuffled: bitwise the same loss rows up to summation order,
+    # checked to the parity tolerance
+    rng = np.random.default_rng(5)
+    perm = rng.permutation(W.E)
+    P2 = DeviceProblem(W.am_scores, W.edges[:, perm].copy(), W.weights[perm].copy(), W.start_end_states, W.seq_lens,
+                       W.n_states)
+    post2, loss2 = P2.run(cabi.OUT_PROB)
+    assert torch.all((loss2 - loss).abs() <= 1e-5 * loss.abs() + 1e-6)
+    assert float((post2 - post).abs().max()) <= 1e-4
+
+
+def test_full_size_best_path(oracle):
+    """Best path on the headline automata: bit-identical to the oracle, and the path's own score,
+    re-accumulated in float64 along the alignment, matches the reported score."""
+    W = make_workload("cart")
+    dev = torch.device("cuda:0")
+    am = torch.from_numpy(-W.am_scores).to(dev)
+    d = dict(edges=torch.from_numpy(W.edges).to(dev), w=torch.from_numpy(-W.weights).to(dev),
+             se=torch.from_numpy(W.start_end_states).to(dev), lens=torch.from_numpy(W.seq_lens).to(dev))
+    align = torch.empty((W.T, W.B), dtype=torch.int32, device=dev)
+    scores = torch.empty((W.B,), dtype=torch.float32, device=dev)
+    nbytes = cabi.workspace_size(W.T, W.B, W.F, W.E, W.n_states)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    cabi.viterbi(am.data_ptr(), am.stride(0), am.stride(1), d["edges"].data_ptr(), d["edges"].stride(0), d["w"].data_ptr(),
+                 d["se"].data_ptr(), d["se"].stride(0), d["lens"].data_ptr(), W.T, W.B, W.F, W.E, W.n_states,
+                 align.data_ptr(), align.stride(0), align.stride(1), scores.data_ptr(), ws.data_ptr(), nbytes, stream)
+    assert cabi.read_status(ws.data_ptr(), W.B, stream) == (0, -1)
+    want_align, want_scores = oracle.viterbi_oracle(-W.am_scores, W.edges, -W.weights, W.start_end_states, W.seq_lens,
+                                                    W.n_states)
+    np.testing.assert_array_equal(align.cpu().numpy(), want_align)
+    np.testing.assert_array_equal(scores.cpu().numpy().view(np.uint32), want_scores.view(np.uint32))
+    # emission scores along the alignment are an upper part of the path score: score - sum(am) = sum of edge weights <= 0
+    a = align.cpu().numpy()
+    for b in range(0, W.B, 8):
+        L = int(W.seq_lens[b])
+        em = float((-W.am_scores[np.arange(L), b, a[:L, b]]).astype(np.float64).sum())
+        assert float(scores[b]) <= em + 1e-3
