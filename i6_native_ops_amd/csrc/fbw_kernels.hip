@@ -454,7 +454,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     };
 
     // sort keys: (primary << 13) | position in input order; ties keep the input order
-    int N = 2;
+    int N = 1024;                       // at least one key per thread, see below
     while (N < n_edges) N <<= 1;
     for (int i = tid; i < N; i += 1024) {
         unsigned k = ~0u;
@@ -466,6 +466,28 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         keys[i] = k;
     }
     __syncthreads();
+    if (N == 1024) {
+        // one key per thread: partners less than a wave apart are reached with a lane exchange, so
+        // only 10 of the 55 compare-exchange steps go through LDS and barriers
+        unsigned x = keys[tid];
+        for (int k = 2; k <= 1024; k <<= 1) {
+            for (int j = k >> 1; j > 0; j >>= 1) {
+                unsigned y;
+                if (j >= 64) {
+                    keys[tid] = x;
+                    __syncthreads();
+                    y = keys[tid ^ j];
+                    __syncthreads();
+                } else {
+                    y = (unsigned)__shfl_xor((int)x, j);
+                }
+                const bool up = (tid & k) == 0, lower = (tid & j) == 0;
+                x = (lower == up) ? min(x, y) : max(x, y);
+            }
+        }
+        keys[tid] = x;
+        __syncthreads();
+    } else
     for (int k = 2; k <= N; k <<= 1) {
         for (int j = k >> 1; j > 0; j >>= 1) {
             for (int i = tid; i < N; i += 1024) {
