@@ -19,6 +19,7 @@ STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
            "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment", "i6fbw_set_band",
+           "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
            "i6fbw_profile_enable", "i6fbw_profile_read")
 
 _lib = None
@@ -54,6 +55,15 @@ def load():
         lib.i6fbw_dump_alignment.restype = c.c_int
         lib.i6fbw_set_band.argtypes = [c.c_int]
         lib.i6fbw_set_band.restype = None
+        lib.i6fbw_ctc_fsa_bounds.argtypes = [c.c_int, c.c_int, c.POINTER(c.c_int), c.POINTER(c.c_int), c.POINTER(c.c_size_t)]
+        lib.i6fbw_ctc_fsa_bounds.restype = c.c_int
+        lib.i6fbw_build_ctc_fsa.argtypes = [c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_void_p, c.c_int64,
+                                            c.c_int, c.c_void_p, c.c_void_p, c.c_int64, c.c_void_p, c.c_void_p, c.c_void_p]
+        lib.i6fbw_build_ctc_fsa.restype = c.c_int
+        lib.i6fbw_build_hmm_fsa.argtypes = [c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_void_p, c.c_float,
+                                            c.c_float, c.c_void_p, c.c_int64, c.c_int, c.c_void_p, c.c_void_p, c.c_int64,
+                                            c.c_void_p, c.c_void_p]
+        lib.i6fbw_build_hmm_fsa.restype = c.c_int
         lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
         lib.i6fbw_read_status.restype = c.c_int
         lib.i6fbw_strerror.argtypes = [c.c_int]
@@ -126,6 +136,34 @@ def read_status(ws_ptr, B, stream=0):
 def set_overlap(mode: int) -> None:
     """-1: by problem size, 0: single stream, 1: overlapped stages."""
     load().i6fbw_set_overlap(int(mode))
+
+
+def ctc_fsa_bounds(B, Lmax):
+    """(edge capacity, state bound, scratch bytes) that always suffice for i6fbw_build_ctc_fsa."""
+    e, n, sb = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
+    rc = load().i6fbw_ctc_fsa_bounds(B, Lmax, ctypes.byref(e), ctypes.byref(n), ctypes.byref(sb))
+    if rc != 0:
+        raise FbwError(rc)
+    return int(e.value), int(n.value), int(sb.value)
+
+
+def build_ctc_fsa(targets_ptr, target_row_stride, target_lens_ptr, B, Lmax, blank, edges_ptr, edge_row_stride, edge_capacity,
+                  weights_ptr, start_end_ptr, se_row_stride, totals_ptr, scratch_ptr, stream=0) -> None:
+    rc = load().i6fbw_build_ctc_fsa(targets_ptr, target_row_stride, target_lens_ptr, B, Lmax, blank, edges_ptr,
+                                    edge_row_stride, edge_capacity, weights_ptr, start_end_ptr, se_row_stride, totals_ptr,
+                                    scratch_ptr, stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def build_hmm_fsa(labels_ptr, label_row_stride, label_lens_ptr, B, Lmax, states_per_label, emission_table_ptr, loop_weight,
+                  forward_weight, edges_ptr, edge_row_stride, edge_capacity, weights_ptr, start_end_ptr, se_row_stride,
+                  totals_ptr, stream=0) -> None:
+    rc = load().i6fbw_build_hmm_fsa(labels_ptr, label_row_stride, label_lens_ptr, B, Lmax, states_per_label,
+                                    emission_table_ptr, loop_weight, forward_weight, edges_ptr, edge_row_stride,
+                                    edge_capacity, weights_ptr, start_end_ptr, se_row_stride, totals_ptr, stream)
+    if rc != 0:
+        raise FbwError(rc)
 
 
 def set_band(on: bool) -> None:

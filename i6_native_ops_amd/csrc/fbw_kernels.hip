@@ -254,8 +254,9 @@ __global__ __launch_bounds__(256) void fbw_scan_sorted(const int32_t* e_seq, int
         const unsigned prev = i > 0 ? (unsigned)e_seq[i - 1] : 0u;
         mybad |= cur < prev;
         // sequences prev+1 .. cur (from 0 for the first edge) start at edge i
+        // (sequence index -1 marks a padding edge; such edges sort behind all others)
         unsigned q0 = i > 0 ? prev + 1u : 0u;
-        if (cur >= q0 && cur != 0xffffffffu)
+        if (!(i > 0 && prev == 0xffffffffu))
             for (unsigned q = q0; q <= min(cur, (unsigned)B); q++) seqbegin[q] = i;
         if (i == E - 1)
             for (unsigned q = min(cur, (unsigned)B) + 1u; q <= (unsigned)B; q++) seqbegin[q] = E;
@@ -344,7 +345,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     if (sorted) {
         edge_begin = E > 0 ? a.seqbegin[b] : 0;
         n_edges = E > 0 ? a.seqbegin[b + 1] - edge_begin : 0;
-        if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B) bad = 1;
+        if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B && (unsigned)e_seq[E - 1] != 0xffffffffu) bad = 1;
         for (int i = edge_begin + tid; i < edge_begin + n_edges; i += 1024) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
             mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
@@ -365,7 +366,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
                 mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
                 if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
             }
-            if (b == 0 && s >= (unsigned)a.B) bad = 1;
+            if (b == 0 && s >= (unsigned)a.B && s != 0xffffffffu) bad = 1;
         }
         if (lt) atomicAdd(&s_lt, lt);
         if (bad) atomicOr(&s_bad, 1);
@@ -1821,3 +1822,4 @@ int i6fbw_profile_read(float* stage_ms) {
 }  // extern "C"
 
 #include "viterbi_kernels.inc"
+#include "fsa_builders.inc"

@@ -58,6 +58,8 @@ int i6fbw_workspace_size(int T, int B, int F, int E, int n_states, size_t* bytes
  *               innermost stride 1                                   (fbw_op.cu:258,268-276)
  *   edges       int32 [4,E] rows from, to, emission_idx, sequence_idx, row stride edge_row_stride
  *                                                                    (fbw_op.cu:249-256)
+ *               An edge with sequence_idx -1 is padding and ignored (an extension: the reference
+ *               has no such value), so an edge list can be handed over at its capacity.
  *   weights     float [E], -log space                                (fbw_op.cu:257)
  *   start_end   int32 [2,B] row 0 start states, row 1 end states, row stride se_row_stride
  *                                                                    (fbw_op.cu:260-263)
@@ -152,6 +154,42 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
  * not depend on the schedule.  No counterpart in the reference.
  */
 void i6fbw_set_overlap(int mode);
+
+/*
+ * Device-side construction of the automaton arrays for two common topologies.  No counterpart in
+ * the reference, which leaves the tuple (number of states, edges, weights, start/end states) to
+ * its callers (fbw/__init__.py:56-62); these take that step off the host.  States of sequence b
+ * are contiguous and follow those of sequence b-1, edges are grouped by sequence.  Edges from the
+ * number actually produced up to edge_capacity are written as padding edges (sequence index -1),
+ * which i6fbw_run and i6fbw_viterbi skip: pass E = edge_capacity and any upper bound of the number
+ * of states as n_states, and the host never needs the exact counts.  totals (device, 2 ints)
+ * receives them anyway: [0] edges produced, [1] states.
+ *
+ * i6fbw_build_ctc_fsa: CTC with the emission on the target state of an edge.  Per sequence with
+ * labels l_1..l_L (targets[b * target_row_stride + i], L = target_lens[b] limited to [0, Lmax]): a
+ * non-emitting start state, the 2L+1 states blank, l_1, blank, ..., l_L, blank and a terminal end
+ * state; loops, edges to the next state, label-to-next-label edges where the labels differ, the
+ * start state feeding the first blank and the first label, and a copy into the terminal state of
+ * every edge that enters the last label or the last blank.  All weights 0.  With these arrays
+ * i6fbw_run's sum_output equals torch.nn.functional.ctc_loss(reduction="none") per sequence.
+ * i6fbw_ctc_fsa_bounds gives capacities that always suffice and the size of `scratch` (device).
+ *
+ * i6fbw_build_hmm_fsa: left-to-right chain, states_per_label states per label, each with a loop
+ * (loop_weight) and an edge to the next state (forward_weight), both emitting
+ * emission_table[label * states_per_label + k] (the index itself if emission_table is NULL): the
+ * emission sits on the source state as in the reference's test (test/fbw.py:28-32); the last state
+ * leads to a non-emitting end state.  Exactly 2 * states_per_label * sum(L) edges and
+ * states_per_label * sum(L) + B states; capacities B * Lmax * states_per_label * 2 and
+ * B * (Lmax * states_per_label + 1) always suffice.  totals may be NULL if edge_capacity is exact.
+ */
+int i6fbw_ctc_fsa_bounds(int B, int Lmax, int* max_edges, int* max_states, size_t* scratch_bytes);
+int i6fbw_build_ctc_fsa(const int32_t* targets, int64_t target_row_stride, const int32_t* target_lens, int B, int Lmax,
+                        int blank, int32_t* edges, int64_t edge_row_stride, int edge_capacity, float* weights,
+                        int32_t* start_end, int64_t se_row_stride, int32_t* totals, void* scratch, void* stream);
+int i6fbw_build_hmm_fsa(const int32_t* labels, int64_t label_row_stride, const int32_t* label_lens, int B, int Lmax,
+                        int states_per_label, const int32_t* emission_table, float loop_weight, float forward_weight,
+                        int32_t* edges, int64_t edge_row_stride, int edge_capacity, float* weights,
+                        int32_t* start_end, int64_t se_row_stride, int32_t* totals, void* stream);
 
 /*
  * Debug dumps of the reference (fbw_op.cu:155-224, switched by DebugOptions, DebugOptions.h:4-9).
