@@ -69,6 +69,7 @@ constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
 constexpr int REC_THREADS_DENSE = 448;
 constexpr int REC_BLOCK_DENSE = REC_THREADS_DENSE + 64 * REC_LOADERS;
 constexpr unsigned NO_STATE = 0xFFFFu;
+constexpr int SEQ_GENERIC = 1;        // value of SeqMeta::err / errA / errB that routes a sequence to the general path
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
 constexpr int SYNC_HDR = 16;          // ints before the progress counters in the hand-off area:
                                       // [0] abort flag, [1] recursion workgroups placed so far, [3] preparation workgroups finished
@@ -90,7 +91,7 @@ struct SeqMeta {
     int err;          // common problems (written by the emission-order role)
     int Kin, errA;    // written by the target-order role
     int Kout, errB;   // written by the source-order role
-    int pad;
+    int pad;          // bit 0: edges contiguous in the input
 };
 
 __host__ __device__ inline long long round16(long long x) { return (x + 15) & ~15LL; }
@@ -138,12 +139,20 @@ __device__ unsigned long long g_trace[4096];   // debug builds only: in-kernel t
 // ---------------------------------------------------------------------------------------------
 // small device helpers
 // ---------------------------------------------------------------------------------------------
-__device__ inline int seq_error(const SeqMeta& m) { return m.err ? m.err : (m.errA ? m.errA : m.errB); }
+// negative: a reported problem; SEQ_GENERIC: handled by the general path; 0: fast path
+__device__ inline int seq_error(const SeqMeta& m) {
+    if (m.err < 0) return m.err;
+    if (m.errA < 0) return m.errA;
+    if (m.errB < 0) return m.errB;
+    return (m.err | m.errA | m.errB) ? 1 : 0;
+}
 
-// Recursion class of a sequence: 0 nothing to do, 1..3 by size, -1 error.
+// Recursion class of a sequence: 0 nothing to do, 1..3 by size, -1 error, -2 general path.
 __device__ inline int rec_class(const SeqMeta& m, const int threads = REC_THREADS) {
-    if (seq_error(m)) return -1;
+    const int err = seq_error(m);
+    if (err < 0) return -1;
     if (m.L == 0 || m.n_edges == 0) return 0;
+    if (err > 0) return -2;            // general path
     if (m.SP <= threads && m.DP <= 512) return 1;
     if (m.SP <= 4 * threads && m.DP <= 2048) return 2;
     return 3;
@@ -170,13 +179,14 @@ template <bool SYNC, typename T> __device__ __forceinline__ T load_x(const T* p)
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // polls *p until it is >= want; false if it gave up (or somebody else already had to)
-__device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort_flag) {
+// (quiet: running out of polls is not an error yet, the caller tries again)
+__device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort_flag, bool quiet = false) {
     for (int n = 0; n < SPIN_LIMIT; n++) {
         if (load_agent(p) >= want) return true;
         if ((n & 255) == 255 && load_agent(abort_flag)) return false;
         __builtin_amdgcn_s_sleep(2);
     }
-    atomicOr(abort_flag, 1);
+    if (!quiet) atomicOr(abort_flag, 1);
     return false;
 }
 
@@ -235,6 +245,7 @@ struct PrepArgs {
     int T, B, F, E, n_states;
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
+    int force_generic;  // F is too large for the emission bitmap or the row image: every sequence takes the general path
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
@@ -379,7 +390,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     unsigned smin = min(min(s_min, st_state), en_state), smax = max(max(s_max, st_state), en_state);
     int err = 0;
     if (s_bad || st_state >= (unsigned)a.n_states || en_state >= (unsigned)a.n_states) err = I6FBW_ERR_BAD_INDEX;
-    else if (n_edges > EB_MAX) err = I6FBW_ERR_SEQ_TOO_MANY_EDGES;
+    // Sequences beyond the capacity of the fast kernels take the general path (see
+    // generic_path.inc); the best-path search has no such path and reports them.
+    const bool gen_ok = !a.best_path;
+    int generic = 0;
+    if (!err && n_edges > EB_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_MANY_EDGES; }
     const unsigned sl = (unsigned)a.seq_lens[b];
     // full sum: a length outside [1, T] leaves the sequence without probability mass; best path:
     // lengths beyond T are read as T
@@ -387,7 +402,8 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     long long S = (long long)smax - smin + 1;
     if (!err && n_edges > 0 && S > 2LL * n_edges + 2) err = I6FBW_ERR_SEQ_SPARSE_STATES;
     if (n_edges == 0) S = 1;
-    if (!err && S > S_MAX) err = I6FBW_ERR_SEQ_TOO_LARGE;
+    if (!err && S > S_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
+    if (!err && a.force_generic && n_edges > 0) generic = 1;
     const int SP = (int)round16(S);
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
@@ -396,12 +412,12 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     auto edge_at = [&](int i) -> int { return sorted ? edge_begin + i : eidx[i]; };
 
     int D = 0;
-    if (!err && n_edges > 0) {
-        if (!sorted) {
-            // stable list of this sequence's edge indices (every role writes the same values)
-            for (int i = lo; i < hi; i++)
-                if ((unsigned)e_seq[i] == (unsigned)b) eidx[pos++] = i;
-        }
+    if (!err && n_edges > 0 && !sorted) {
+        // stable list of this sequence's edge indices (every role writes the same values)
+        for (int i = lo; i < hi; i++)
+            if ((unsigned)e_seq[i] == (unsigned)b) eidx[pos++] = i;
+    }
+    if (!err && !generic && n_edges > 0) {
         // emission presence bitmap -> slot = rank of the emission id among the distinct ones
         const int nwords = (a.F + 31) >> 5;
         for (int w = tid; w < nwords; w += 1024) bitmap[w] = 0u;
@@ -418,7 +434,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         int run = block_excl_scan(c, wsum, 16, &D);
         for (int w = w0; w < w1; w++) { wordpfx[w] = run; run += __popc(bitmap[w]); }
         __syncthreads();
-        if (D > D_MAX) err = I6FBW_ERR_SEQ_TOO_LARGE;
+        if (D > D_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
@@ -434,9 +450,10 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         m->edge_begin = edge_begin; m->n_edges = n_edges; m->state_min = (int)smin;
         m->S = (int)S; m->SP = SP; m->D = D; m->DP = DP; m->L = L;
         m->start_local = (int)(st_state - smin); m->end_local = (int)(en_state - smin);
-        m->err = err; m->pad = 0;
+        m->err = err ? err : (generic ? SEQ_GENERIC : 0);
+        m->pad = sorted ? 1 : 0;         // bit 0: the edges of the sequence are contiguous in the input
     }
-    if (err || n_edges == 0) {
+    if (err || generic || n_edges == 0) {
         if (tid == 0) {
             if (role == 0) { a.meta[b].Kin = 0; a.meta[b].errA = 0; }
             if (role == 1) { a.meta[b].Kout = 0; a.meta[b].errB = 0; }
@@ -517,7 +534,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         if (kmax) atomicMax(&s_kmax, kmax);
         __syncthreads();
         const int K = s_kmax;
-        const int kerr = K > KMAX ? I6FBW_ERR_SEQ_DEGREE : 0;
+        const int kerr = K > KMAX ? (gen_ok ? SEQ_GENERIC : I6FBW_ERR_SEQ_DEGREE) : 0;
         if (tid == 0) {
             if (role == 0) { a.meta[b].Kin = K; a.meta[b].errA = kerr; }
             else { a.meta[b].Kout = K; a.meta[b].errB = kerr; }
@@ -673,7 +690,10 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
 // With SYNC the loader wave waits for the gather flags, the rows are written through, and the
 // number of finished rows is published every PUBLISH steps for the combine kernel.
 // ---------------------------------------------------------------------------------------------
+#include "generic_path.inc"
+
 struct RecArgs {
+    GenArgs gen;
     int T, B;
     int prep_wgs;     // workgroups of the preparation kernel
     const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab;
@@ -989,7 +1009,7 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     float (*amr)[D_MAX] = (float (*)[D_MAX])lds;
     float (*st)[S_MAX + 16] = (float (*)[S_MAX + 16])(lds + 2 * D_MAX);
     float* wmin = lds + 2 * D_MAX + 2 * (S_MAX + 16);
-    int* go_flag = (int*)(wmin + 8);
+    int* go_flag = (int*)(wmin + 32);      // wmin doubles as the 32-float scratch of the general path's reductions
 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
     // gather or combine waves
@@ -1009,6 +1029,12 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     const int b = blockIdx.x >> 1, dir = blockIdx.x & 1;
     const SeqMeta m = a.meta[b];
     const int cls = rec_class(m, T_);
+    if (cls == -2) {
+        const long long soff = state_off(m.edge_begin, b);
+        generic_recurse<SYNC>(a.gen, m, b, dir, a.T, (dir ? a.beta : a.alpha) + (size_t)a.T * soff,
+                              (dir ? a.offB : a.offA) + (size_t)b * a.T, a.sync + SYNC_HDR + 2 * b + dir, wmin);
+        return;
+    }
     if (cls <= 0) return;
     const bool loader = threadIdx.x >= T_;
     const int K = dir ? m.Kout : m.Kin;
@@ -1033,7 +1059,7 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     }
 }
 
-constexpr int REC_LDS_FLOATS = 2 * D_MAX + 2 * (S_MAX + 16) + 8 + 8;
+constexpr int REC_LDS_FLOATS = 2 * D_MAX + 2 * (S_MAX + 16) + 32 + 8;
 template <bool SYNC>
 __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS];
@@ -1054,6 +1080,7 @@ __global__ __launch_bounds__(REC_BLOCK_DENSE, 5) void fbw_recurse_dense(RecArgs 
 // filled once and only those positions are rewritten per frame before the row is streamed out.
 // ---------------------------------------------------------------------------------------------
 struct CombArgs {
+    GenArgs gen;
     int T, B, F, out_mode;
     const SeqMeta* meta; const uint4* crec; const int* cbegin; const int* demis;
     const float* alpha; const float* beta; const float* gtab; const double* offA; const double* offB;
@@ -1159,7 +1186,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
 #ifdef I6_TRACE
     if (tid == 0) { atomicMin(&g_trace[2], wall_clock64()); if (b == 0) g_trace[1024 + strip] = wall_clock64(); }
 #endif
-    if (seq_error(m) || m.n_edges == 0) {
+    if (seq_error(m) < 0 || m.n_edges == 0) {
         // no recursion ran for this sequence: NaN for a reported problem, empty frames otherwise
         const bool err = seq_error(m) != 0;
         const float v = err ? __builtin_nanf("") : (a.out_mode != I6FBW_OUT_NEG_LOG ? 0.f : INF_F);
@@ -1177,13 +1204,23 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             // the gather strips of these frames, then both recursions
             bool ok = true;
             const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG);
-            for (int g = t0 / TG; ok && g <= (tv - 1) / TG; g++) ok = spin_until_ge(gflag + g, 1, a.sync);
-            ok = ok && spin_until_ge(prog, tv, a.sync);
-            ok = ok && spin_until_ge(prog + 1, m.L - t0, a.sync);
+            const bool general = seq_error(m) > 0;      // no gather for it, and a recursion that takes its time
+            for (int g = t0 / TG; !general && ok && g <= (tv - 1) / TG; g++) ok = spin_until_ge(gflag + g, 1, a.sync);
+            for (int rep = 0; rep < (general ? 64 : 1); rep++) {
+                ok = spin_until_ge(prog, tv, a.sync, general && rep < 63) && spin_until_ge(prog + 1, m.L - t0, a.sync, general && rep < 63);
+                if (ok || load_agent(a.sync)) break;
+            }
             s_ok = ok;
         }
         __syncthreads();
         if (!s_ok) return;       // timed out: reported through the abort flag
+    }
+    if (seq_error(m) > 0) {
+        __shared__ float gred[32];
+        const long long soff = state_off(m.edge_begin, b);
+        generic_combine<SYNC>(a.gen, m, b, t0, tv, T, B, F, a.out_mode, a.alpha + (size_t)T * soff, a.beta + (size_t)T * soff,
+                              a.offA + (size_t)b * T, a.offB + (size_t)b * T, a.out, a.ost_t, a.ost_b, a.sum_output, gred);
+        return;
     }
     const bool prob = a.out_mode != I6FBW_OUT_NEG_LOG;
     const float hole = prob ? 0.f : INF_F;
@@ -1523,7 +1560,10 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
     const Layout l = make_layout(T, B, E);
     if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
-    if (F > F_BITMAP_MAX || comb_lds_bytes(F) > 160 * 1024 - 256) return I6FBW_ERR_F_TOO_LARGE;
+    // too many emission classes for the LDS bitmap of the preparation or the LDS row image of the
+    // dense write: every sequence takes the general path
+    const bool f_too_large = F > F_BITMAP_MAX || comb_lds_bytes(F) > 160 * 1024 - 256;
+    const size_t comb_lds = f_too_large ? 64 : comb_lds_bytes(F);
 
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
@@ -1558,7 +1598,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
-    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = g_no_band;
+    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = g_no_band; pa.force_generic = f_too_large ? 1 : 0;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
@@ -1566,11 +1606,16 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
     ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.per_group = per_group;
+    GenArgs gen;
+    gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
+    gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx;
     RecArgs ra;
+    ra.gen = gen;
     ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
     ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.sync = sync;
     CombArgs ca;
+    ca.gen = gen;
     ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
@@ -1634,7 +1679,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
         { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS, s, ra);
           else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
+        { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
         HIP_TRY(hipGetLastError());
         return I6FBW_OK;
     }
@@ -1656,7 +1701,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
 #ifdef I6_TRACE
     if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
 #endif
-    { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds_bytes(F), s, ca); }
+    { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
     HIP_TRY(hipGetLastError());
     // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
@@ -1678,7 +1723,8 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
     if (e != hipSuccess) { g_last_hip_error = e; free(host); return I6FBW_ERR_LAUNCH; }
     *code = aborted ? I6FBW_ERR_TIMEOUT : I6FBW_OK; *seq = -1;
     for (int b = 0; b < B; b++) {
-        const int c = host[b].err ? host[b].err : (host[b].errA ? host[b].errA : host[b].errB);
+        // positive values mark sequences that took the general path
+        const int c = host[b].err < 0 ? host[b].err : (host[b].errA < 0 ? host[b].errA : (host[b].errB < 0 ? host[b].errB : 0));
         if (c) { *code = c; *seq = b; break; }
     }
     free(host);

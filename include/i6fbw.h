@@ -25,11 +25,16 @@ enum {
     I6FBW_ERR_INVALID_ARGUMENT = -1,   /* null pointer, non-positive T/B/F/n_states, bad out_mode */
     I6FBW_ERR_WORKSPACE_TOO_SMALL = -2,
     I6FBW_ERR_LAUNCH = -3,             /* a HIP launch failed; see i6fbw_last_hip_error() */
-    I6FBW_ERR_F_TOO_LARGE = -4,        /* F beyond what the row image / emission bitmap hold */
-    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* device-side: one sequence has more edges than supported */
-    I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* device-side: state ids of one sequence span more than 2*edges+2 */
-    I6FBW_ERR_SEQ_DEGREE = -12,           /* device-side: a state has more in- or out-edges than supported */
-    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side: states / distinct emissions of one sequence exceed LDS */
+    /* The four size codes are reported by i6fbw_viterbi only.  i6fbw_run takes sequences beyond
+       these sizes (more than 8192 edges, 4096 states or 4096 distinct emissions in one sequence,
+       more than 8 edges into or out of a state, F beyond about 36 000) through a general path that
+       has no such limits and runs at a fraction of the speed. */
+    I6FBW_ERR_F_TOO_LARGE = -4,           /* F beyond what the emission bitmap holds (131 072) */
+    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* device-side: one sequence has more than 8192 edges */
+    I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* device-side: state ids of one sequence span more than 2*edges+2
+                                             (i6fbw_run too: the workspace is sized by the edge count) */
+    I6FBW_ERR_SEQ_DEGREE = -12,           /* device-side: a state has more than 8 incoming edges */
+    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side: more than 4096 states / distinct emissions in one sequence */
     I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
     I6FBW_ERR_TIMEOUT = -15               /* device-side: a stage gave up waiting for another stage of the call */
 };

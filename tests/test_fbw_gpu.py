@@ -14,7 +14,7 @@ LOSS_RTOL = 1e-5
 POST_ATOL = 1e-4
 
 
-def check_against_oracle(oracle, args, threads=1):
+def check_against_oracle(oracle, args, threads=1, bitwise=True):
     from i6_native_ops_amd import cabi
     from tests.gpu_util import run_cabi
     am, edges, weights, start_end, seq_lens, n_states = args
@@ -27,7 +27,10 @@ def check_against_oracle(oracle, args, threads=1):
     # holes are +inf in exactly the same places (a posterior below float range may differ)
     assert (np.isposinf(out) | (want_post < 1e-30) == np.isposinf(want_out) | (want_post < 1e-30)).all()
     prob, loss2 = run_cabi(*args, out_mode=cabi.OUT_PROB)
-    np.testing.assert_array_equal(loss2, loss)
+    if bitwise:      # the fast kernels sum in a fixed order; the general path accumulates with atomics
+        np.testing.assert_array_equal(loss2, loss)
+    else:
+        np.testing.assert_allclose(loss2, loss, rtol=1e-6)
     np.testing.assert_allclose(prob, want_post, rtol=0, atol=POST_ATOL)
     assert (prob[np.isposinf(want_out)] == 0).all()
     return out, loss

@@ -1,0 +1,79 @@
+"""Automata beyond the capacity of the fast kernels (more than 8 edges into or out of a state,
+more than 8192 edges, 4096 states or 4096 distinct emissions in one sequence, more emission
+classes than the LDS row image holds) take the general path inside the same kernels.  Same parity
+bar as everything else, under both schedules, also mixed with ordinary sequences in one batch."""
+import numpy as np
+import pytest
+
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.test_fbw_gpu import check_against_oracle, schedule  # noqa: F401  (autouse fixture: both schedules)
+
+pytestmark = pytest.mark.gpu
+
+
+def fan(rng, T, F, n_mid, seq=0, off=0):
+    """start -> n_mid parallel middle states -> end, every middle state with a loop: degree n_mid at
+    the start (out) and at the end (in)."""
+    frm, to, emis = [], [], []
+    s, e = off, off + n_mid + 1
+    for i in range(n_mid):
+        mid = off + 1 + i
+        frm += [s, mid, mid]
+        to += [mid, mid, e]
+        emis += [int(x) for x in rng.integers(0, F, size=3)]
+    n = len(frm)
+    edges = np.array([frm, to, emis, [seq] * n], dtype=np.int32)
+    return edges, rng.uniform(0.0, 1.5, size=n).astype(np.float32), s, e, n_mid + 2
+
+
+def test_high_degree_mixed_with_ordinary_sequences(oracle):
+    rng = np.random.default_rng(11)
+    W = make_workload("tiny")                                  # two ordinary sequences ...
+    T, F = W.T, W.F
+    e2, w2, s2, t2, n2 = fan(rng, T, F, 20, seq=2, off=W.n_states)          # ... and one with degree 20
+    edges = np.concatenate([W.edges, e2], axis=1)
+    weights = np.concatenate([W.weights, w2])
+    start_end = np.concatenate([W.start_end_states, np.array([[s2], [t2]], np.int32)], axis=1)
+    seq_lens = np.concatenate([W.seq_lens, np.array([17], np.int32)])
+    am = rng.uniform(0.1, 4.0, size=(T, 3, F)).astype(np.float32)
+    am[:, :2] = W.am_scores
+    for shuffle in (False, True):
+        if shuffle:
+            perm = rng.permutation(edges.shape[1])
+            edges, weights = edges[:, perm].copy(), weights[perm].copy()
+        check_against_oracle(oracle, (am, edges, weights, start_end, seq_lens, W.n_states + n2), bitwise=False)
+
+
+@pytest.mark.parametrize("kind", ["many_states", "many_edges", "many_emissions"])
+def test_large_sequences(oracle, kind):
+    """Left-to-right chains beyond one of the per-sequence capacities."""
+    if kind == "many_states":       # 4500 states, 9000 edges
+        W = make_workload("cart", T=9000, B=1, F=300, n_labels=(1500, 1500))
+        W.seq_lens[:] = W.T
+    elif kind == "many_edges":      # silence states add edges: > 8192 edges with < 4096 states is not reachable with
+        W = make_workload("longform", T=8400, B=2, F=700, n_labels=(1380, 1390))   # chains, so this also has > 4096 states
+        W.seq_lens[:] = W.T
+    else:                           # 4200 distinct emissions among 1400 labels x 3 states
+        W = make_workload("cart", T=8400, B=1, F=50000, n_labels=(1400, 1400))
+        W.seq_lens[:] = W.T
+    per_seq = W.edges_per_seq()
+    print(kind, "edges per sequence", per_seq.tolist(), "states", W.n_states, flush=True)
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=4, bitwise=False)
+
+
+@pytest.mark.parametrize("F", [40000, 140000])
+def test_many_emission_classes(oracle, F):
+    """F beyond the LDS row image (about 36 000) and beyond the emission bitmap (131 072): all sequences
+    take the general path."""
+    W = make_workload("cart", T=60, B=3, F=F, n_labels=(10, 15))
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), bitwise=False)
+
+
+def test_status_is_clean_for_general_path():
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import DeviceProblem
+    rng = np.random.default_rng(2)
+    edges, weights, s, e, n = fan(rng, 12, 9, 30)
+    am = rng.uniform(0.1, 3.0, size=(12, 1, 9)).astype(np.float32)
+    P = DeviceProblem(am, edges, weights, np.array([[s], [e]], np.int32), np.array([12], np.int32), n)
+    P.run(cabi.OUT_PROB)                 # raises on any reported status

@@ -110,10 +110,17 @@ def test_device_side_status_is_reported():
     bad[3, 0] = 3                       # sequence index >= B
     with pytest.raises(RuntimeError, match="index out of range"):
         core.fbw(am, bad, weights, se, seq_lens, n)
-    # a state with 9 incoming edges
+    # state ids of one sequence spread over far more ids than it has edges
+    sparse = edges.clone()
+    sparse[1, 1] = 40
+    sparse[0, 2] = 40
+    sparse[1, 2] = 40
+    with pytest.raises(RuntimeError, match="span more than"):
+        core.fbw(am, sparse, weights, torch.tensor([[0], [40]], dtype=torch.int32, device="cuda"), seq_lens, 41)
+    # a state with 9 incoming edges is beyond the fast kernels, not beyond the library
     many = torch.tensor([[0] * 9, [1] * 9, [0] * 9, [0] * 9], dtype=torch.int32, device="cuda")
-    with pytest.raises(RuntimeError, match="more than 8 incoming or outgoing edges"):
-        core.fbw(am, many, torch.zeros(9, device="cuda"), se, seq_lens, n)
+    out, loss = core.fbw(am, many, torch.zeros(9, device="cuda"), se, torch.tensor([1], dtype=torch.int32, device="cuda"), n)
+    assert torch.isfinite(loss[0]).all() and (loss[1:] == 0).all()
     # the good input still works afterwards
     out, loss = core.fbw(am, edges, weights, se, seq_lens, n)
     assert torch.isfinite(loss).all()
