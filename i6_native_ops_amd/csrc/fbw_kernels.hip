@@ -1585,6 +1585,11 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
     if (2 * B > 2 * P.n_cu) overlap = false;
+    if (overlap) {
+        // under stream capture: one stream, no in-memory waits between kernels, no synchronisation
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) overlap = false;
+    }
     if (overlap) { int rc = runs_beside(P, s, &overlap); if (rc != I6FBW_OK) return rc; }
     hipStream_t sP = overlap ? P.sP : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;

@@ -165,3 +165,31 @@ def test_fused_fbw_loss_equals_unfused_wrapper_and_oracle(oracle, name, kw, over
         np.testing.assert_array_equal(loss.detach().cpu().numpy(), results[0][0])
     finally:
         cabi.set_overlap(-1)
+
+
+def test_graph_capture_of_a_large_call(oracle):
+    """A call big enough for the overlapped schedule, captured into a HIP graph: the library then
+    stays on the capturing stream (no library streams, no in-memory waits, no synchronisation), and
+    every replay gives the eager result."""
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import DeviceProblem
+    W = make_workload("cart", T=400, B=16, F=12001)            # T*B*F > 2^26
+    P = DeviceProblem(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    eager_post, eager_loss = P.run(cabi.OUT_PROB)
+    eager_post, eager_loss = eager_post.clone(), eager_loss.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        P.run(cabi.OUT_PROB, check=False)                      # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            P.run(cabi.OUT_PROB, check=False)
+    for _ in range(3):
+        P.out.fill_(-1.0)
+        P.loss.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(P.loss, eager_loss)
+        assert torch.equal(P.out, eager_post)
