@@ -42,16 +42,7 @@ constexpr int D_MAX = 4096;           // distinct emissions of one sequence
 #ifndef I6_TG
 #define I6_TG 8
 #endif
-#ifndef I6_GATHER_BFAST
-#define I6_GATHER_BFAST 0
-#endif
 constexpr int TG = I6_TG;             // frames per gather workgroup
-#ifndef I6_P1
-#define I6_P1 8
-#endif
-#ifndef I6_REC_PAD_LDS
-#define I6_REC_PAD_LDS 0
-#endif
 #ifndef I6_TC
 #define I6_TC 8
 #endif
@@ -190,17 +181,11 @@ __device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort
     return false;
 }
 
-// Order in which gather and combine workgroups are handed out (1-D grid, dispatched in index
-// order): the batch is cut into `groups` blocks of `per_group` sequences, and a block goes through
-// all of its strips before the next block starts.  The first block's recursions then reach the
-// middle of their sequences, where the dense write can begin, after 1/groups of the gather, and
-// the gather of the later blocks runs beside the dense write of the earlier ones.
-__device__ __forceinline__ void grouped_index(int per_group, int n_strips, int B, int* b, int* y) {
-    const int bi = blockIdx.x % per_group;
-    const int rest = blockIdx.x / per_group;
-    *y = rest % n_strips;
-    *b = (rest / n_strips) * per_group + bi;
-    if (*b >= B) *b = -1;
+// Gather and combine workgroups are handed out (1-D grid, dispatched in index order) with the
+// sequence index running fastest: workgroups that run together read / write neighbouring rows.
+__device__ __forceinline__ void strip_index(int B, int* b, int* y) {
+    *b = blockIdx.x % B;
+    *y = blockIdx.x / B;
 }
 
 // wave-wide minimum in lane 63 (DPP row operations, no LDS traffic)
@@ -390,9 +375,9 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     unsigned smin = min(min(s_min, st_state), en_state), smax = max(max(s_max, st_state), en_state);
     int err = 0;
     if (s_bad || st_state >= (unsigned)a.n_states || en_state >= (unsigned)a.n_states) err = I6FBW_ERR_BAD_INDEX;
-    // Sequences beyond the capacity of the fast kernels take the general path (see
-    // generic_path.inc); the best-path search has no such path and reports them.
-    const bool gen_ok = !a.best_path;
+    // Sequences beyond the capacity of the fast kernels take the general path (generic_path.inc,
+    // generic_viterbi).
+    constexpr bool gen_ok = true;
     int generic = 0;
     if (!err && n_edges > EB_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_MANY_EDGES; }
     const unsigned sl = (unsigned)a.seq_lens[b];
@@ -640,14 +625,12 @@ struct GatherArgs {
     const SeqMeta* meta; const int* demis; const int2* tband; float* gtab;
     int* sync;
     float scale;      // log2(e) for -log scores, -log2(e) for log scores
-    int per_group;    // sequences per block of the hand-out order
 };
 
 template <bool SYNC>
 __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
     int b, y;
-    grouped_index(a.per_group, (a.T + TG - 1) / TG, a.B, &b, &y);
-    if (b < 0) return;
+    strip_index(a.B, &b, &y);
     const SeqMeta m = a.meta[b];
     if (rec_class(m) <= 0) return;
     const int n = (m.L + TG - 1) / TG;
@@ -770,11 +753,7 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
         const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
         stn[s] = r;
-#ifdef I6_HACK_SPARSE_STORES
-        if (s < SP && (i & 3) == 0) store_x<SYNC>(cur.wp + s, r);
-#else
         if (s < SP) store_x<SYNC>(cur.wp + s, r);
-#endif
         rmin = fminf(rmin, r);
     }
     if (tid == 0) store_x<SYNC>(cur.op, cur.c);
@@ -1041,7 +1020,7 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     if (cls == 1) {
-        if (loader) recurse_load<SYNC, T_, 4, (DENSE ? 8 : I6_P1)>(a, m, b, dir, amr[0], amr[1]);
+        if (loader) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
         else if (K <= 2) recurse_compute<SYNC, T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
@@ -1087,7 +1066,6 @@ struct CombArgs {
     float* out; float* sum_output;
     long long ost_t, ost_b;      // element strides of out over frames and sequences
     int* sync;
-    int per_group;               // sequences per block of the hand-out order
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1171,8 +1149,7 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     // write neighbouring rows
     const int tid = threadIdx.x;
     int b, y;
-    grouped_index(a.per_group, (a.T + TC - 1) / TC, a.B, &b, &y);
-    if (b < 0) return;
+    strip_index(a.B, &b, &y);
     const SeqMeta m = a.meta[b];
     if (m.L == 0) return;                                      // fbw_padfill has written every row
     const int T = a.T, B = a.B, F = a.F;
@@ -1415,7 +1392,6 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_padfill(const int32_t* seq_l
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-constexpr int MAX_CHUNKS = 32;
 constexpr int MAX_DEVICES = 64;
 
 thread_local hipError_t g_last_hip_error = hipSuccess;
@@ -1515,12 +1491,6 @@ struct StageTimer {
 size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
-int g_groups = [] {
-    // blocks of sequences in the overlapped schedule; more than one lets the dense write start before
-    // the gather is over, which measured slower (the kernels get in each other's way), so the default is 1
-    const char* e = getenv("I6FBW_GROUPS");
-    return e ? atoi(e) : 0;
-}();
 int g_no_band = 0;      // see i6fbw_set_band
 int g_overlap_mode = [] {
     const char* e = getenv("I6FBW_OVERLAP");
@@ -1594,12 +1564,9 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     hipStream_t sP = overlap ? P.sP : s, sR = overlap ? P.sR : s;
     if (g_prof.on) g_prof.n_calls++;
 
-    // blocks of sequences for the hand-out order of gather and combine (see grouped_index)
-    const int groups = overlap ? std::max(1, std::min(g_groups > 0 ? g_groups : 1, B / 8)) : 1;
-    const int per_group = (B + groups - 1) / groups;
-    const dim3 g_grid((unsigned)(per_group * groups) * ((T + TG - 1) / TG)), c_grid((unsigned)(per_group * groups) * ((T + TC - 1) / TC));
+    const dim3 g_grid((unsigned)B * ((T + TG - 1) / TG)), c_grid((unsigned)B * ((T + TC - 1) / TC));
     const dim3 p_grid(B, (T + TC - 1) / TC);
-    if ((long long)per_group * groups * ((T + TG - 1) / TG) > 0x7fffffffLL) return I6FBW_ERR_INVALID_ARGUMENT;
+    if ((long long)B * ((T + TG - 1) / TG) > 0x7fffffffLL) return I6FBW_ERR_INVALID_ARGUMENT;
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
@@ -1610,7 +1577,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
-    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.per_group = per_group;
+    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E;
     GenArgs gen;
     gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
     gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx;
@@ -1624,7 +1591,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ca.T = T; ca.B = B; ca.F = F; ca.out_mode = out_mode;
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
-    ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync; ca.per_group = per_group;
+    ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
 
     {
@@ -1694,10 +1661,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // held back until every recursion workgroup is on the machine -- normally long since.
     hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
     HIP_TRY(hipGetLastError());
-#ifndef I6_GATHER_LDS
-#define I6_GATHER_LDS 0
-#endif
-    { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), I6_GATHER_LDS, s, ga); }
+    { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, s, ga); }
     HIP_TRY(hipGetLastError());
     // The dense write follows the gather on the same stream (its workgroups would only take wave
     // slots away from the gather before that: by then the two recursions are about to meet in the

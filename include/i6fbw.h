@@ -25,16 +25,19 @@ enum {
     I6FBW_ERR_INVALID_ARGUMENT = -1,   /* null pointer, non-positive T/B/F/n_states, bad out_mode */
     I6FBW_ERR_WORKSPACE_TOO_SMALL = -2,
     I6FBW_ERR_LAUNCH = -3,             /* a HIP launch failed; see i6fbw_last_hip_error() */
-    /* The four size codes are reported by i6fbw_viterbi only.  i6fbw_run takes sequences beyond
-       these sizes (more than 8192 edges, 4096 states or 4096 distinct emissions in one sequence,
-       more than 8 edges into or out of a state, F beyond about 36 000) through a general path that
-       has no such limits and runs at a fraction of the speed. */
-    I6FBW_ERR_F_TOO_LARGE = -4,           /* F beyond what the emission bitmap holds (131 072) */
-    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* device-side: one sequence has more than 8192 edges */
+    /* Sequences beyond the capacity of the fast kernels (more than 8192 edges, 4096 states or 4096
+       distinct emissions in one sequence, more than 8 edges into or out of a state, F beyond about
+       36 000 for i6fbw_run / 131 072 for i6fbw_viterbi) are not refused: they take a general path
+       that has no such limits and runs at a fraction of the speed.  The size codes remain for the
+       one case that path cannot hold either. */
+    I6FBW_ERR_F_TOO_LARGE = -4,           /* not returned any more */
+    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* not reported any more */
     I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* device-side: state ids of one sequence span more than 2*edges+2
-                                             (i6fbw_run too: the workspace is sized by the edge count) */
-    I6FBW_ERR_SEQ_DEGREE = -12,           /* device-side: a state has more than 8 incoming edges */
-    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side: more than 4096 states / distinct emissions in one sequence */
+                                             (the workspace is sized by the edge count) */
+    I6FBW_ERR_SEQ_DEGREE = -12,           /* not reported any more */
+    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side, i6fbw_viterbi: values and back-pointers of a sequence on the
+                                             general path do not fit its share of the workspace (T < 2*edges+16 with
+                                             state ids spread over nearly 2*edges ids) */
     I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
     I6FBW_ERR_TIMEOUT = -15               /* device-side: a stage gave up waiting for another stage of the call */
 };
@@ -140,7 +143,8 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
  * decides them, so alignment and scores equal the reference's bit for bit.  seq_lens[b] > T
  * (undefined in the reference) is read as T.  One kernel chain on `stream`; per-sequence
  * problems are reported by i6fbw_read_status, the affected sequences get score NaN and an
- * all-zero alignment.
+ * all-zero alignment.  Sequences beyond the capacity of the fast kernel run the reference's own
+ * scheme (per-frame sweeps over the edge list with atomics) and give the same bits.
  */
 int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
                   const int32_t* edges, int64_t edge_row_stride,

@@ -113,13 +113,45 @@ def test_size_classes(oracle, kind):
 
 
 def test_device_status():
-    """A state with more than eight incoming edges is reported, its sequence gets score NaN and zeros."""
-    n = 10
-    edges = np.array([[s, n, s % 3, 0] for s in range(n)] + [[0, s, 1, 0] for s in range(1, n)], dtype=np.int32).T.copy()
+    """State ids spread over far more ids than the sequence has edges are reported; the sequence gets
+    score NaN and an all-zero alignment."""
+    edges = np.array([[0, 50, 1, 0], [50, 50, 2, 0]], dtype=np.int32).T.copy()
     am = np.zeros((2, 1, 4), dtype=np.float32)
-    a, s, code = run_cabi_viterbi(am, edges, np.zeros(edges.shape[1], np.float32), np.array([[0], [n]], np.int32),
-                                  np.array([2], np.int32), n + 1, check=False)
-    assert code == -12 and np.isnan(s[0]) and (a == 0).all()
+    a, s, code = run_cabi_viterbi(am, edges, np.zeros(2, np.float32), np.array([[0], [50]], np.int32),
+                                  np.array([2], np.int32), 51, check=False)
+    assert code == -11 and np.isnan(s[0]) and (a == 0).all()
+
+
+@pytest.mark.parametrize("kind", ["degree", "many_states", "many_classes", "ties"])
+def test_general_path(oracle, kind):
+    """Beyond the capacity of the fast kernels (more than 8 edges into a state, more than 4096 states,
+    more emission classes than the bitmap holds): same bits as the oracle, ties included."""
+    rng = np.random.default_rng(77)
+    if kind in ("degree", "ties"):
+        T, F, n_mid = 14, 9, 25
+        frm, to, emis = [], [], []
+        for i in range(n_mid):
+            frm += [0, 1 + i, 1 + i]
+            to += [1 + i, 1 + i, n_mid + 1]
+            emis += [int(x) for x in rng.integers(0, F, size=3)]
+        edges = np.array([frm, to, emis, [0] * len(frm)], dtype=np.int32)
+        weights = rng.uniform(-1.5, 0.0, size=len(frm)).astype(np.float32)
+        am = -rng.uniform(0.1, 3.0, size=(T, 1, F)).astype(np.float32)
+        if kind == "ties":
+            weights[:] = -0.5
+            am = np.round(am)
+        args = (am, edges, weights, np.array([[0], [n_mid + 1]], np.int32), np.array([11], np.int32), n_mid + 2)
+    elif kind == "many_states":
+        W = make_workload("cart", T=5000, B=1, F=300, n_labels=(1500, 1500))
+        W.seq_lens[:] = W.T
+        args = (-W.am_scores, W.edges, -W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    else:
+        W = make_workload("cart", T=60, B=3, F=140000, n_labels=(10, 15))
+        args = (-W.am_scores, W.edges, -W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    got = run_cabi_viterbi(*args)[:2]
+    want = oracle.viterbi_oracle(*args)
+    assert np.isfinite(want[1]).all()
+    assert_identical(got, want)
 
 
 def test_python_interface(oracle):
