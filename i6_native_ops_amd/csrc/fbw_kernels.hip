@@ -1108,11 +1108,10 @@ __device__ inline void stream_image_row(float* row, int F, const float4a* lds4, 
     constexpr int U = 4;                                        // LDS reads in flight per thread
     for (int c0 = threadIdx.x; c0 < ch_hi; c0 += U * COMB_THREADS) {
         float4a v[U];
+        // no branch around the reads (the compiler would wait for each one before the next):
+        // chunks past the end re-read the last one and are not stored
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int ch = c0 + u * COMB_THREADS;
-            if (ch < ch_hi) v[u] = lds4[ch];
-        }
+        for (int u = 0; u < U; u++) v[u] = lds4[min(c0 + u * COMB_THREADS, ch_hi - 1)];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int ch = c0 + u * COMB_THREADS;
