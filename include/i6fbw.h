@@ -78,9 +78,11 @@ int i6fbw_workspace_size(int T, int B, int F, int E, int n_states, size_t* bytes
  *               t < seq_lens[b], 0 elsewhere                         (fbw_op.cu:104-135,232)
  *   workspace   device buffer of at least i6fbw_workspace_size bytes, 256-byte aligned
  *   stream      hipStream_t to enqueue on (NULL = default stream); the call is asynchronous.
- *               Inside, the work forks onto library-owned streams (created on first use, default
- *               priority) and joins `stream` again before the call returns, so everything
- *               enqueued on `stream` afterwards sees the finished outputs.
+ *               Inside, a large call forks onto library-owned streams (created on first use,
+ *               default priority) and joins `stream` again before the call returns, so everything
+ *               enqueued on `stream` afterwards sees the finished outputs.  The first large call
+ *               on a stream synchronises it once (a check that the library's streams run beside
+ *               it); under stream capture the call stays on `stream` and can be replayed.
  *
  * Returns I6FBW_OK or a negative host-side status.  Problems only the device can
  * see (index out of range, an automaton beyond the supported size) are recorded in
