@@ -18,6 +18,11 @@
 // t+1 == seq_len (fbw_op.cu:61-69), edge score +inf if either side is +inf (fbw_op.cu:83-86),
 // sum_output = 0 for empty frames (fbw_op.cu:120-128), out = +inf where nothing contributes
 // (fbw_op.cu:41-44,131-134,152,366-369).
+//
+// Parts of this translation unit: this file (kernels of the four stages, the host side of
+// i6fbw_run, status, dumps), generic_path.inc (sequences beyond the capacity of those kernels),
+// viterbi_kernels.inc (best path on the same tables, i6fbw_viterbi), fsa_builders.inc (CTC / HMM
+// automaton arrays built on the device).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
