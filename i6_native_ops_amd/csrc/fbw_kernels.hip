@@ -630,6 +630,7 @@ struct GatherArgs {
     const SeqMeta* meta; const int* demis; const int2* tband; float* gtab;
     int* sync;
     float scale;      // log2(e) for -log scores, -log2(e) for log scores
+    int ascending;    // strips in ascending order (one consumer walking forward) instead of from both ends inwards
 };
 
 template <bool SYNC>
@@ -640,7 +641,7 @@ __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
     if (rec_class(m) <= 0) return;
     const int n = (m.L + TG - 1) / TG;
     if (y >= n) return;
-    const int j = (y & 1) ? n - 1 - (y >> 1) : (y >> 1);
+    const int j = a.ascending ? y : ((y & 1) ? n - 1 - (y >> 1) : (y >> 1));
     const int t0 = j * TG;
     const long long goff = slot_off(m.edge_begin, b);
     const int* de = a.demis + goff;
@@ -1581,7 +1582,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
-    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E;
+    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.ascending = 0;
     GenArgs gen;
     gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
     gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx;

@@ -143,7 +143,8 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
  * Values are computed in the reference's arithmetic, (previous + weight) + score in fp32, and
  * ties go to the edge that comes first in the input, as the reference's compare-and-swap rule
  * decides them, so alignment and scores equal the reference's bit for bit.  seq_lens[b] > T
- * (undefined in the reference) is read as T.  One kernel chain on `stream`; per-sequence
+ * (undefined in the reference) is read as T.  Asynchronous on `stream` (large problems use the
+ * library's stream beside it, as i6fbw_run does, and join `stream` before returning); per-sequence
  * problems are reported by i6fbw_read_status, the affected sequences get score NaN and an
  * all-zero alignment.  Sequences beyond the capacity of the fast kernel run the reference's own
  * scheme (per-frame sweeps over the edge list with atomics) and give the same bits.

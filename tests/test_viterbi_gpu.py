@@ -14,6 +14,14 @@ from tests.test_oracle_viterbi import viterbi_fixture
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["single_stream", "overlapped"], autouse=True)
+def schedule(request):
+    """Every case runs under both schedules of i6fbw_viterbi (search after / beside the gather)."""
+    cabi.set_overlap(0 if request.param == "single_stream" else 1)
+    yield request.param
+    cabi.set_overlap(-1)
+
+
 def run_cabi_viterbi(am, edges, weights, start_end, seq_lens, n_states, check=True):
     dev = torch.device("cuda:0")
     T, B, F = am.shape
