@@ -1685,20 +1685,21 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
 
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq) {
     if (!workspace || B <= 0 || !code || !seq) return I6FBW_ERR_INVALID_ARGUMENT;
-    SeqMeta* host = (SeqMeta*)malloc(sizeof(SeqMeta) * (size_t)B);
+    // the meta records sit at the start of the workspace, the abort flag of the hand-off area right
+    // behind them: one copy brings both
+    const size_t flag_at = align256(sizeof(SeqMeta) * (size_t)B);
+    char* host = (char*)malloc(flag_at + sizeof(int));
     if (!host) return I6FBW_ERR_INVALID_ARGUMENT;
-    // the meta records sit at the start of the workspace
-    hipError_t e = hipMemcpyAsync(host, workspace, sizeof(SeqMeta) * (size_t)B, hipMemcpyDeviceToHost, (hipStream_t)stream);
+    hipError_t e = hipMemcpyAsync(host, workspace, flag_at + sizeof(int), hipMemcpyDeviceToHost, (hipStream_t)stream);
     if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
     if (e != hipSuccess) { g_last_hip_error = e; free(host); return I6FBW_ERR_LAUNCH; }
     int aborted = 0;
-    // the abort flag of the hand-off area follows the meta records
-    e = hipMemcpy(&aborted, (const char*)workspace + align256(sizeof(SeqMeta) * (size_t)B), sizeof(int), hipMemcpyDeviceToHost);
-    if (e != hipSuccess) { g_last_hip_error = e; free(host); return I6FBW_ERR_LAUNCH; }
+    memcpy(&aborted, host + flag_at, sizeof(int));
+    const SeqMeta* meta = (const SeqMeta*)host;
     *code = aborted ? I6FBW_ERR_TIMEOUT : I6FBW_OK; *seq = -1;
     for (int b = 0; b < B; b++) {
         // positive values mark sequences that took the general path
-        const int c = host[b].err < 0 ? host[b].err : (host[b].errA < 0 ? host[b].errA : (host[b].errB < 0 ? host[b].errB : 0));
+        const int c = meta[b].err < 0 ? meta[b].err : (meta[b].errA < 0 ? meta[b].errA : (meta[b].errB < 0 ? meta[b].errB : 0));
         if (c) { *code = c; *seq = b; break; }
     }
     free(host);
