@@ -1603,7 +1603,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
         // the scan also clears the header of the hand-off area, so it runs even without edges
         StageTimer tm(0, s);
         hipLaunchKernelGGL(fbw_scan_sorted, dim3(std::max(1, (E + SCAN_BLOCK - 1) / SCAN_BLOCK)), dim3(256), 0, s,
-                           edges + 3 * edge_row_stride, E, B, pa.sortflag, pa.seqbegin, sync);
+                           E > 0 ? edges + 3 * edge_row_stride : nullptr, E, B, pa.sortflag, pa.seqbegin, sync);
         HIP_TRY(hipGetLastError());
     }
     // Where the recursion kernel is started: beside the preparation if its 2B workgroups leave at
