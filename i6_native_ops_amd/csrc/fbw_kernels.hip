@@ -727,8 +727,14 @@ __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
 
 // One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
 // LDS, log-sum-exp (base 2) in a fixed order, result to the other LDS buffer and the workspace.
-template <bool SYNC, int THREADS, int J, int KT>
-__device__ __forceinline__ void recurse_step(const int i, const int SP, const char* stc, float* stn,
+template <typename ST> __device__ __forceinline__ ST state_min(ST a, ST b) { return b < a ? b : a; }
+
+// ST is the type of the state vector in LDS: float, or double for sequences whose alignment is so
+// constrained that the states carrying the posterior mass sit far from the frame minimum (their
+// values would lose precision in float, frame after frame).  exp2 / log2 always work in float on
+// differences, which are small; rows go to the workspace as float either way.
+template <bool SYNC, int THREADS, int J, int KT, typename ST>
+__device__ __forceinline__ void recurse_step(const int i, const int SP, const char* stc, ST* stn,
                                              const char* amc, float* wmin,
                                              const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
                                              const float (&ew)[J][KT], RecCursor& cur) {
@@ -746,21 +752,21 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
 #pragma unroll
     for (int j = 0; j < J; j++) {
         const int s = tid + j * THREADS;
-        float v[KT];
-        float mn = INF_F;
+        ST v[KT];
+        ST mn = (ST)INF_F;
 #pragma unroll
         for (int k = 0; k < KT; k++) {
-            v[k] = *(const float*)(stc + eo[j][k]) + (ew[j][k] + *(const float*)(amc + es[j][k]));
-            mn = fminf(mn, v[k]);
+            v[k] = *(const ST*)(stc + eo[j][k]) + (ST)(ew[j][k] + *(const float*)(amc + es[j][k]));
+            mn = state_min(mn, v[k]);
         }
         float sum = 0.f;
 #pragma unroll
-        for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f(mn - v[k]);
+        for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f((float)(mn - v[k]));
         // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
-        const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
+        const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
         stn[s] = r;
-        if (s < SP) store_x<SYNC>(cur.wp + s, r);
-        rmin = fminf(rmin, r);
+        if (s < SP) store_x<SYNC>(cur.wp + s, (float)r);
+        rmin = fminf(rmin, (float)r);
     }
     if (tid == 0) store_x<SYNC>(cur.op, cur.c);
     cur.wp += cur.wstep; cur.op += cur.ostep;
@@ -773,9 +779,9 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
 }
 
 // common prologue of the compute waves: initial state vector, row 0 of the workspace, cursor
-template <bool SYNC, int THREADS>
+template <bool SYNC, int THREADS, typename ST>
 __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int SCAP,
-                                             float* st0, float* st1, RecCursor& cur) {
+                                             ST* st0, ST* st1, RecCursor& cur) {
     const int tid = threadIdx.x;
     const int L = m.L, SP = m.SP, T = a.T;
     const long long soff = state_off(m.edge_begin, b);
@@ -806,9 +812,9 @@ __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m,
     if (SYNC && tid == 0) store_agent(cur.progress, 1);      // the initial row is out
 }
 
-template <bool SYNC, int THREADS, int J, int KT>
+template <bool SYNC, int THREADS, int J, int KT, typename ST>
 __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                                float* st0, float* st1,
+                                                ST* st0, ST* st1,
                                                 const float* am0, const float* am1,
                                                 float* wmin) {
     constexpr int SCAP = THREADS * J;
@@ -830,25 +836,25 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
             if (k < K && s < SP) r = ell[(size_t)k * SP + s];
             unsigned other = r.x & 0xFFFFu;
             if (other == NO_STATE) other = SCAP;          // LDS cell that always holds +inf
-            eo[j][k] = other * 4u;
+            eo[j][k] = other * (unsigned)sizeof(ST);
             es[j][k] = (r.x >> 16) * 4u;
             ew[j][k] = __uint_as_float(r.y);
         }
     }
     RecCursor cur;
-    recurse_init<SYNC, THREADS>(a, m, b, dir, SCAP, st0, st1, cur);
+    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
     for (int i = 0; i < cur.nsteps; i += 2) {
-        recurse_step<SYNC, THREADS, J, KT>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
+        recurse_step<SYNC, THREADS, J, KT, ST>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
         if (i + 1 < cur.nsteps)
-            recurse_step<SYNC, THREADS, J, KT>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
+            recurse_step<SYNC, THREADS, J, KT, ST>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
     }
 }
 
 // Fallback for the largest sequences: same arithmetic, edge tables re-read from memory each frame
 // instead of living in registers.
-template <bool SYNC, int THREADS>
+template <bool SYNC, int THREADS, typename ST>
 __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                                        float* st0, float* st1,
+                                                        ST* st0, ST* st1,
                                                         const float* am0, const float* am1,
                                                         float* wmin, const int SCAP) {
     constexpr int NW = THREADS / 64;
@@ -858,8 +864,8 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
     const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
     const int K = dir ? m.Kout : m.Kin;
     RecCursor cur;
-    recurse_init<SYNC, THREADS>(a, m, b, dir, SCAP, st0, st1, cur);
-    float* stc = st0; float* stn = st1;
+    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
+    ST* stc = st0; ST* stn = st1;
     const float* amc = am0; const float* amn = am1;
     for (int i = 0; i < cur.nsteps; i++) {
         float pend = 0.f;
@@ -872,25 +878,25 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
         }
         float rmin = INF_F;
         for (int s = tid; s < SP; s += THREADS) {
-            float v[KMAX];
-            float mn = INF_F;
+            ST v[KMAX];
+            ST mn = (ST)INF_F;
 #pragma unroll
             for (int k = 0; k < KMAX; k++) {
-                v[k] = INF_F;
+                v[k] = (ST)INF_F;
                 if (k < K) {
                     const uint2 r = ell[(size_t)k * SP + s];
                     const unsigned other = r.x & 0xFFFFu;
-                    if (other != NO_STATE) v[k] = stc[other] + (__uint_as_float(r.y) + amc[r.x >> 16]);
-                    mn = fminf(mn, v[k]);
+                    if (other != NO_STATE) v[k] = stc[other] + (ST)(__uint_as_float(r.y) + amc[r.x >> 16]);
+                    mn = state_min(mn, v[k]);
                 }
             }
             float sum = 0.f;
 #pragma unroll
-            for (int k = 0; k < KMAX; k++) sum += __builtin_amdgcn_exp2f(mn - v[k]);
-            const float r = mn == INF_F ? INF_F : (mn - pend) - __builtin_amdgcn_logf(sum);
+            for (int k = 0; k < KMAX; k++) sum += __builtin_amdgcn_exp2f((float)(mn - v[k]));
+            const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
             stn[s] = r;
-            store_x<SYNC>(cur.wp + s, r);
-            rmin = fminf(rmin, r);
+            store_x<SYNC>(cur.wp + s, (float)r);
+            rmin = fminf(rmin, (float)r);
         }
         if (tid == 0) store_x<SYNC>(cur.op, cur.c);
         cur.wp += cur.wstep; cur.op += cur.ostep;
@@ -900,7 +906,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
             if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
         }
         step_end<SYNC>(i, cur);
-        float* t_ = stc; stc = stn; stn = t_;
+        ST* t_ = stc; stc = stn; stn = t_;
         const float* u_ = amc; amc = amn; amn = u_;
     }
 }
@@ -987,13 +993,43 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
 // the gate, gather and combine waves need to get onto the unit at all.
 // The host picks it when the batch has more workgroups than the device has compute units.  The rarely used large-automaton paths pay for the cap with spills,
 // which is why small batches run the uncapped instance.
+// LDS of a recursion workgroup, in floats: two emission rows, two state vectors (of doubles in
+// the uncapped instance, see recurse_step), per-wave minima / reduction scratch, a flag.
+constexpr int REC_LDS_FLOATS_F32 = 2 * D_MAX + 2 * (S_MAX + 16) + 32 + 8;
+constexpr int REC_LDS_FLOATS_F64 = 2 * D_MAX + 4 * (S_MAX + 16) + 32 + 8;
+
+// the compute threads' part for one state type; the loader waves do not depend on it
+template <bool SYNC, int T_, typename ST>
+__device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int cls,
+                                                 ST* st0, ST* st1, const float* am0, const float* am1, float* wmin) {
+    const int K = dir ? m.Kout : m.Kin;
+    // The loop body is specialised on the number of states per thread and of edge slots per state,
+    // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
+    // (Fewer specialisations for double: it is the rare case.)
+    constexpr bool F32 = sizeof(ST) == 4;
+    if (cls == 1) {
+        if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (F32 && K <= 3) recurse_compute<SYNC, T_, 1, F32 ? 3 : 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (F32 && K <= 6) recurse_compute<SYNC, T_, 1, F32 ? 6 : KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else recurse_compute<SYNC, T_, 1, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+    } else if (cls == 2) {
+        if (K <= 2) recurse_compute<SYNC, T_, 4, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (F32 && K <= 3) recurse_compute<SYNC, T_, 4, F32 ? 3 : 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (K <= 4) recurse_compute<SYNC, T_, 4, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, 4 * T_);
+    } else {
+        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
+    }
+}
+
 template <bool SYNC, bool DENSE>
 __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) {
     constexpr int T_ = DENSE ? REC_THREADS_DENSE : REC_THREADS;
-    // LDS of a workgroup (REC_LDS_FLOATS floats, 16-byte aligned): the emission rows first
+    // LDS of a workgroup (16-byte aligned): the emission rows first
     float (*amr)[D_MAX] = (float (*)[D_MAX])lds;
-    float (*st)[S_MAX + 16] = (float (*)[S_MAX + 16])(lds + 2 * D_MAX);
-    float* wmin = lds + 2 * D_MAX + 2 * (S_MAX + 16);
+    float* stf = lds + 2 * D_MAX;                                        // state vectors, float or double
+    float* wmin = stf + (DENSE ? 2 : 4) * (S_MAX + 16);
     int* go_flag = (int*)(wmin + 32);      // wmin doubles as the 32-float scratch of the general path's reductions
 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
@@ -1021,36 +1057,31 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
         return;
     }
     if (cls <= 0) return;
-    const bool loader = threadIdx.x >= T_;
-    const int K = dir ? m.Kout : m.Kin;
-    // The loop body is specialised on the number of states per thread and of edge slots per state,
-    // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
-    if (cls == 1) {
-        if (loader) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
-        else if (K <= 2) recurse_compute<SYNC, T_, 1, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 3) recurse_compute<SYNC, T_, 1, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 4) recurse_compute<SYNC, T_, 1, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 6) recurse_compute<SYNC, T_, 1, 6>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else recurse_compute<SYNC, T_, 1, KMAX>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-    } else if (cls == 2) {
-        if (loader) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1]);
-        else if (K <= 2) recurse_compute<SYNC, T_, 4, 2>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 3) recurse_compute<SYNC, T_, 4, 3>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else if (K <= 4) recurse_compute<SYNC, T_, 4, 4>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin);
-        else recurse_compute_generic<SYNC, T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, 4 * T_);
+    if (threadIdx.x >= T_) {
+        if (cls == 1) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
+        else if (cls == 2) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1]);
+        else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
+        return;
+    }
+    // Double-precision state vectors where a sequence has fewer than five frames for every three
+    // states: there the alignment is constrained enough for float to show (measured: 1100 states
+    // in 1055 frames reach 1.4e-4 on the posteriors in float).  The dense instance has no room for
+    // them in LDS.
+    const bool wide = !DENSE && 5LL * m.S > 3LL * m.L;
+    if (wide) {
+        double* st0 = (double*)stf;
+        recurse_dispatch<SYNC, T_, double>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);
     } else {
-        if (loader) recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
-        else recurse_compute_generic<SYNC, T_>(a, m, b, dir, st[0], st[1], amr[0], amr[1], wmin, S_MAX);
+        recurse_dispatch<SYNC, T_, float>(a, m, b, dir, cls, stf, stf + (S_MAX + 16), amr[0], amr[1], wmin);
     }
 }
 
-constexpr int REC_LDS_FLOATS = 2 * D_MAX + 2 * (S_MAX + 16) + 32 + 8;
 template <bool SYNC>
 __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
-    __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS_F64];
     recurse_workgroup<SYNC, false>(a, lds);
 }
-// The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS floats): with the
+// The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS_F32 floats): with the
 // size known at compile time the compiler sees that at most two workgroups fit on a unit anyway
 // and ignores the register cap, and two workgroups then fill the register file.
 template <bool SYNC>
@@ -1433,8 +1464,8 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
     for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
-        HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS));
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS));
+        HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     p.ready = true;
@@ -1611,7 +1642,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // LDS and could otherwise find no room while the recursion waits for them), else behind it.
     const bool early = overlap && 2 * B <= P.n_cu / 2;
     auto launch_recursion = [&]() -> int {
-        { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS, sR, ra);
+        { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
           else hipLaunchKernelGGL(fbw_recurse<true>, dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
         HIP_TRY(hipGetLastError());
         HIP_TRY(hipEventRecord(P.doneR, sR));
@@ -1653,7 +1684,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     if (!overlap) {
         { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS, s, ra);
+        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, s, ra);
           else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
         { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }

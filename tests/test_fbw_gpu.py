@@ -63,6 +63,14 @@ def test_random_automata_brute_force(oracle, seed):
     np.testing.assert_allclose(posterior(out), want_post, atol=POST_ATOL)
 
 
+def test_tightly_constrained_alignment(oracle):
+    """About one frame per state over more than a thousand states: the states that carry the posterior
+    mass sit far from the frame minimum; the recursion keeps such sequences in double precision."""
+    W = make_workload("cart", T=1150, B=3, F=400, n_labels=(366, 370))
+    W.seq_lens[:] = [1150, 1120, 1135]
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=3)
+
+
 @pytest.mark.parametrize("name,kw", [
     ("tiny", {}),
     ("tiny", dict(shuffle_edges=True)),
