@@ -685,7 +685,7 @@ struct RecArgs {
     GenArgs gen;
     int T, B;
     int prep_wgs;     // workgroups of the preparation kernel
-    const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab;
+    const SeqMeta* meta; const uint2* ellA; const uint2* ellB; const float* gtab; float* gtab_rw;
     float* alpha; float* beta; double* offA; double* offB;
     int* sync;
 };
@@ -1052,8 +1052,18 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     const int cls = rec_class(m, T_);
     if (cls == -2) {
         const long long soff = state_off(m.edge_begin, b);
-        generic_recurse<SYNC>(a.gen, m, b, dir, a.T, (dir ? a.beta : a.alpha) + (size_t)a.T * soff,
-                              (dir ? a.offB : a.offA) + (size_t)b * a.T, a.sync + SYNC_HDR + 2 * b + dir, wmin);
+        float* rows = (dir ? a.beta : a.alpha) + (size_t)a.T * soff;
+        double* offs = (dir ? a.offB : a.offA) + (size_t)b * a.T;
+        int* progress = a.sync + SYNC_HDR + 2 * b + dir;
+        // the sequence's share of the compact emission table is unused on this path: room for the
+        // two double-precision working vectors of each direction, unless T is tiny
+        const long long goff = slot_off(m.edge_begin, b);
+        const long long room = (long long)a.T * (slot_off(m.edge_begin + m.n_edges, b + 1) - goff) / 2;      // in doubles
+        if (room >= 4LL * m.SP)
+            generic_recurse_f64<SYNC>(a.gen, m, b, dir, a.T, rows, offs, progress, wmin,
+                                      (double*)(a.gtab_rw + (size_t)a.T * goff) + (size_t)dir * 2 * m.SP);
+        else
+            generic_recurse<SYNC>(a.gen, m, b, dir, a.T, rows, offs, progress, wmin);
         return;
     }
     if (cls <= 0) return;
@@ -1619,7 +1629,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx;
     RecArgs ra;
     ra.gen = gen;
-    ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab;
+    ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab; ra.gtab_rw = ga.gtab;
     ra.alpha = (float*)(ws + l.alpha); ra.beta = (float*)(ws + l.beta);
     ra.offA = (double*)(ws + l.offA); ra.offB = (double*)(ws + l.offB); ra.sync = sync;
     CombArgs ca;

@@ -48,7 +48,7 @@ def test_high_degree_mixed_with_ordinary_sequences(oracle):
 def test_large_sequences(oracle, kind):
     """Left-to-right chains beyond one of the per-sequence capacities."""
     if kind == "many_states":       # 4500 states, 9000 edges
-        W = make_workload("cart", T=9000, B=1, F=300, n_labels=(1500, 1500))
+        W = make_workload("cart", T=7500, B=1, F=300, n_labels=(1500, 1500))
         W.seq_lens[:] = W.T
     elif kind == "many_edges":      # silence states add edges: > 8192 edges with < 4096 states is not reachable with
         W = make_workload("longform", T=8400, B=2, F=700, n_labels=(1380, 1390))   # chains, so this also has > 4096 states
