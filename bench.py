@@ -124,7 +124,7 @@ def main():
             traffic = int(float(m.group(1)) * 1e6)
 
     result = {
-        "metric": "FBW loss+grad ms/call + achieved HBM GB/s at T=1000,B=32,F=12001 fp32",
+        "metric": f"FBW loss+grad ms/call + achieved HBM GB/s at T={W.T},B={W.B},F={W.F} fp32",
         "value": round(gbps, 2),
         "unit": "GB/s",
         "n_gpus": 1,
