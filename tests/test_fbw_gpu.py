@@ -92,3 +92,27 @@ def test_workloads_small(oracle, name, kw):
     W = make_workload(name, **kw)
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states),
                          threads=8)
+
+
+def test_empty_and_minimal_inputs(oracle):
+    """No edges at all, a sequence without edges beside ordinary ones, and the smallest possible problem."""
+    from tests.test_viterbi_gpu import run_cabi_viterbi
+    rng = np.random.default_rng(4)
+    # E = 0: every frame is empty
+    am = rng.uniform(0.1, 3.0, size=(4, 2, 3)).astype(np.float32)
+    none = (am, np.zeros((4, 0), np.int32), np.zeros(0, np.float32), np.array([[0, 1], [0, 2]], np.int32),
+            np.array([4, 2], np.int32), 3)
+    out, loss = check_against_oracle(oracle, none)
+    assert (loss == 0).all() and np.isposinf(out).all()
+    a, s, code = run_cabi_viterbi(-am, *none[1:])
+    assert code == 0 and (a == 0).all() and s.tolist() == [-np.inf, -np.inf]
+    # one sequence of the batch has no edges
+    W = make_workload("tiny")
+    keep = W.edges[3] == 0
+    check_against_oracle(oracle, (W.am_scores, W.edges[:, keep].copy(), W.weights[keep].copy(), W.start_end_states,
+                                  W.seq_lens, W.n_states))
+    # T = B = F = 1, one self-loop on the start = end state
+    one = (np.array([[[0.25]]], np.float32), np.array([[0], [0], [0], [0]], np.int32), np.array([0.5], np.float32),
+           np.array([[0], [0]], np.int32), np.array([1], np.int32), 1)
+    out, loss = check_against_oracle(oracle, one)
+    assert loss[0, 0] == pytest.approx(0.75) and out[0, 0, 0] == pytest.approx(0.0, abs=1e-6)
