@@ -1073,11 +1073,12 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
         else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
         return;
     }
-    // Double-precision state vectors where a sequence has fewer than five frames for every three
-    // states: there the alignment is constrained enough for float to show (measured: 1100 states
-    // in 1055 frames reach 1.4e-4 on the posteriors in float).  The dense instance has no room for
-    // them in LDS.
-    const bool wide = !DENSE && 5LL * m.S > 3LL * m.L;
+    // Double-precision state vectors where float would show in the posteriors: sequences with fewer
+    // than five frames for every three states (the alignment is so constrained that the states
+    // which matter sit far from the frame minimum; 1100 states in 1055 frames reach 1.4e-4 in
+    // float) and sequences of more than 4096 frames (rounding accumulates from frame to frame;
+    // 20 000 frames reach 3e-4 in float).  The dense instance has no room for them in LDS.
+    const bool wide = !DENSE && (5LL * m.S > 3LL * m.L || m.L > 4096);
     if (wide) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);

@@ -116,3 +116,10 @@ def test_empty_and_minimal_inputs(oracle):
            np.array([[0], [0]], np.int32), np.array([1], np.int32), 1)
     out, loss = check_against_oracle(oracle, one)
     assert loss[0, 0] == pytest.approx(0.75) and out[0, 0, 0] == pytest.approx(0.0, abs=1e-6)
+
+
+def test_long_sequences(oracle):
+    """Twenty thousand frames through a short chain: many renormalisations and progress publications."""
+    W = make_workload("monophone", T=20000, B=2, F=120, n_labels=(30, 40))
+    W.seq_lens[:] = [20000, 17333]
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=2)
