@@ -1601,7 +1601,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     bool overlap = forced >= 0 ? forced != 0 : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu);
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
-    if (2 * B > 2 * P.n_cu) overlap = false;
+    if (2 * B > (T <= 4096 ? 2 : 1) * P.n_cu) overlap = false;
     if (overlap) {
         // under stream capture: one stream, no in-memory waits between kernels, no synchronisation
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -1639,7 +1639,10 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
-    const bool dense = 2 * B > P.n_cu;      // more recursion workgroups than compute units
+    // More recursion workgroups than compute units: the instance of which two fit on a unit -- unless
+    // the sequences can be longer than 4096 frames, which only the other instance runs in double
+    // precision (recurse_workgroup); it then takes two rounds.
+    const bool dense = 2 * B > P.n_cu && T <= 4096;
 
     {
         // the scan also clears the header of the hand-off area, so it runs even without edges

@@ -79,6 +79,7 @@ def test_tightly_constrained_alignment(oracle):
     ("monophone", dict(shuffle_edges=True, seed=5)),
     ("cart", dict(T=120, B=4, F=500)),
     ("cart", dict(T=300, B=3, F=12001, shuffle_edges=True)),
+    ("cart", dict(T=40, B=2, F=38000, n_labels=(8, 12))),     # the largest row images that fit into LDS
     ("ctc", dict(T=40, B=8, F=50)),
     ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
     ("ctc", dict(T=30, B=200, F=40)),          # 400 recursion workgroups: two per compute unit, started behind the preparation
@@ -123,3 +124,25 @@ def test_long_sequences(oracle):
     W = make_workload("monophone", T=20000, B=2, F=120, n_labels=(30, 40))
     W.seq_lens[:] = [20000, 17333]
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=2)
+
+
+def test_zero_probability_emissions(oracle):
+    """am_scores = +inf (probability 0) on some emissions, on whole frames of one emission, and on a
+    whole frame: mass flows around them or the sequence has none."""
+    W = make_workload("monophone", T=60, B=4, F=40, n_labels=(4, 6))
+    am = W.am_scores.copy()
+    rng = np.random.default_rng(8)
+    mask = rng.random(am.shape) < 0.05
+    am[mask] = np.inf
+    am[:, 1, 3] = np.inf                      # one emission never possible in sequence 1
+    am[10, 2, :] = np.inf                     # nothing possible in frame 10 of sequence 2: no path at all
+    out, loss = check_against_oracle(oracle, (am, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states))
+    assert (loss[:, 2] == 0).all()
+
+
+def test_large_batch_of_long_sequences(oracle):
+    """More recursion workgroups than compute units and more than 4096 frames: runs on the instance that
+    keeps long sequences in double precision."""
+    W = make_workload("monophone", T=5000, B=140, F=30, n_labels=(3, 5))
+    W.seq_lens[:] = np.random.default_rng(1).integers(4200, 5001, size=140)
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
