@@ -146,3 +146,12 @@ def test_large_batch_of_long_sequences(oracle):
     W = make_workload("monophone", T=5000, B=140, F=30, n_labels=(3, 5))
     W.seq_lens[:] = np.random.default_rng(1).integers(4200, 5001, size=140)
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
+
+
+def test_fast_path_at_capacity(oracle):
+    """4096 states and 8190 edges in one sequence: the most the fast kernels hold (one more label and the
+    sequence takes the general path)."""
+    W = make_workload("cart", T=6200, B=1, F=300, n_labels=(1365, 1365))
+    assert W.n_states == 4096 and W.E == 8190
+    W.seq_lens[:] = W.T
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=1)
