@@ -1185,6 +1185,31 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+// Sum of xs[c0, c1), every lane with a range of its own; called by whole waves.  Ranges of up to
+// LONG_SLOT entries are summed by their lane.  Longer ones (the blank label of a CTC automaton,
+// silence: one emission class on a large share of the edges) would keep one lane busy for
+// microseconds per frame while the rest of the workgroup waits: the wave sums them together, 64
+// entries at a time, in a fixed order.
+constexpr int LONG_SLOT = 16;
+__device__ __forceinline__ float slot_sum(const float* xs, const int c0, const int c1) {
+    const int lane = threadIdx.x & 63;
+    const bool is_long = c1 - c0 > LONG_SLOT;
+    float s = 0.f;
+    if (!is_long)
+        for (int i = c0; i < c1; i++) s += xs[i];
+    unsigned long long todo = __ballot(is_long);
+    while (todo) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int b0 = __builtin_amdgcn_readlane(c0, src), b1 = __builtin_amdgcn_readlane(c1, src);
+        float p = 0.f;
+        for (int q = b0 + lane; q < b1; q += 64) p += xs[q];
+        p = lane63(wave_sum_dpp(p));
+        if (lane == src) s = p;
+    }
+    return s;
+}
+
 template <bool SYNC>
 __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
@@ -1345,10 +1370,8 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
             float lsum = 0.f;
 #pragma unroll
             for (int js = 0; js < JS; js++) {
-                float s = 0.f;
-                for (int i = c0[js]; i < c1[js]; i++) s += xs[i];
-                sd[js] = s;
-                lsum += s;
+                sd[js] = slot_sum(xs, c0[js], c1[js]);
+                lsum += sd[js];
             }
             const float tot = block_sum256(lsum, redsum);
             finish_row(t, mn, tot, sd, em, JS, offs);
@@ -1380,12 +1403,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
 #pragma unroll
                 for (int jd = 0; jd < COMB_JD; jd++) {
                     const int d = tid + jd * COMB_THREADS;
-                    if (d < D) {
-                        const int e0 = max(cb[d], p0), e1 = min(cb[d + 1], p1);
-                        float s = sd[jd];
-                        for (int i = e0; i < e1; i++) s += xs[i - p0];
-                        sd[jd] = s;
-                    }
+                    int e0 = 0, e1 = 0;
+                    if (d < D) { e0 = max(cb[d], p0) - p0; e1 = min(cb[d + 1], p1) - p0; }
+                    sd[jd] += slot_sum(xs, e0, e1);
                 }
             }
             float lsum = 0.f;
