@@ -314,11 +314,13 @@ __device__ inline int min_steps(int from, int to, int dmax, int dmin) {
 // state (beta), role 2 by emission slot (combine) and writes the shared part of the meta record.
 // For edge lists grouped by sequence (the usual case) the scan kernel has recorded where each
 // sequence starts; any other order is handled by a stable scan over the whole list.
-__device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
-    __shared__ unsigned keys[EB_MAX];
-    __shared__ unsigned bitmap[F_BITMAP_MAX / 32];
-    __shared__ int wordpfx[F_BITMAP_MAX / 32];
-    __shared__ int wsum[16];
+template <int NT>
+__device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* lds) {
+    // dynamic LDS: sort keys, then the emission bitmap and its prefix counts (one word per 32 classes)
+    unsigned* keys = lds;
+    unsigned* bitmap = lds + EB_MAX;
+    int* wordpfx = (int*)(bitmap + ((a.F + 31) >> 5));
+    __shared__ int wsum[NT / 64];
     __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin;
     __shared__ unsigned s_min, s_max;
 
@@ -333,7 +335,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     __syncthreads();
     const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
     int unsorted = 0;
-    for (int i = tid; i < nflag; i += 1024) unsorted |= !a.sortflag[i];
+    for (int i = tid; i < nflag; i += NT) unsorted |= !a.sortflag[i];
     if (unsorted) atomicAnd(&s_sorted, 0);
     __syncthreads();
     const bool sorted = s_sorted != 0;
@@ -341,13 +343,13 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     int edge_begin, n_edges, pos = 0;
     int bad = 0;
     unsigned mn = 0xffffffffu, mx = 0u;
-    const int chunk = (E + 1023) / 1024;
+    const int chunk = (E + NT - 1) / NT;
     const int lo = min(E, tid * chunk), hi = min(E, lo + chunk);
     if (sorted) {
         edge_begin = E > 0 ? a.seqbegin[b] : 0;
         n_edges = E > 0 ? a.seqbegin[b + 1] - edge_begin : 0;
         if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B && (unsigned)e_seq[E - 1] != 0xffffffffu) bad = 1;
-        for (int i = edge_begin + tid; i < edge_begin + n_edges; i += 1024) {
+        for (int i = edge_begin + tid; i < edge_begin + n_edges; i += NT) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
             mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
             if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
@@ -372,7 +374,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         if (lt) atomicAdd(&s_lt, lt);
         if (bad) atomicOr(&s_bad, 1);
         if (eq) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
-        pos = block_excl_scan(eq, wsum, 16, &n_edges);   // barriers inside publish the atomics too
+        pos = block_excl_scan(eq, wsum, NT / 64, &n_edges);   // barriers inside publish the atomics too
         edge_begin = s_lt;
     }
 
@@ -410,18 +412,18 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     if (!err && !generic && n_edges > 0) {
         // emission presence bitmap -> slot = rank of the emission id among the distinct ones
         const int nwords = (a.F + 31) >> 5;
-        for (int w = tid; w < nwords; w += 1024) bitmap[w] = 0u;
+        for (int w = tid; w < nwords; w += NT) bitmap[w] = 0u;
         __syncthreads();
-        for (int i = tid; i < n_edges; i += 1024) {
+        for (int i = tid; i < n_edges; i += NT) {
             unsigned em = (unsigned)e_emis[edge_at(i)];
             atomicOr(&bitmap[em >> 5], 1u << (em & 31));
         }
         __syncthreads();
-        const int wpt = (nwords + 1023) / 1024;
+        const int wpt = (nwords + NT - 1) / NT;
         const int w0 = min(nwords, tid * wpt), w1 = min(nwords, w0 + wpt);
         int c = 0;
         for (int w = w0; w < w1; w++) c += __popc(bitmap[w]);
-        int run = block_excl_scan(c, wsum, 16, &D);
+        int run = block_excl_scan(c, wsum, NT / 64, &D);
         for (int w = w0; w < w1; w++) { wordpfx[w] = run; run += __popc(bitmap[w]); }
         __syncthreads();
         if (D > D_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
@@ -433,7 +435,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         const int nstrip = (a.T + TG - 1) / TG;
         if (tid < 2) a.sync[SYNC_HDR + 2 * b + tid] = 0;
         int* gf = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * nstrip;
-        for (int i = tid; i < nstrip; i += 1024) gf[i] = 0;
+        for (int i = tid; i < nstrip; i += NT) gf[i] = 0;
     }
     if (role == 2 && tid == 0) {
         SeqMeta* m = a.meta + b;
@@ -462,9 +464,9 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     };
 
     // sort keys: (primary << 13) | position in input order; ties keep the input order
-    int N = 1024;                       // at least one key per thread, see below
+    int N = NT;                       // at least one key per thread, see below
     while (N < n_edges) N <<= 1;
-    for (int i = tid; i < N; i += 1024) {
+    for (int i = tid; i < N; i += NT) {
         unsigned k = ~0u;
         if (i < n_edges) {
             int e = edge_at(i);
@@ -474,11 +476,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         keys[i] = k;
     }
     __syncthreads();
-    if (N == 1024) {
+    if (N == NT) {
         // one key per thread: partners less than a wave apart are reached with a lane exchange, so
         // only 10 of the 55 compare-exchange steps go through LDS and barriers
         unsigned x = keys[tid];
-        for (int k = 2; k <= 1024; k <<= 1) {
+        for (int k = 2; k <= NT; k <<= 1) {
             for (int j = k >> 1; j > 0; j >>= 1) {
                 unsigned y;
                 if (j >= 64) {
@@ -498,7 +500,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     } else
     for (int k = 2; k <= N; k <<= 1) {
         for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = tid; i < N; i += 1024) {
+            for (int i = tid; i < N; i += NT) {
                 int ixj = i ^ j;
                 if (ixj > i) {
                     unsigned x = keys[i], y = keys[ixj];
@@ -517,7 +519,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         // NO_STATE.
         uint2* ell = (role == 0 ? a.ellA : a.ellB) + (size_t)KMAX * soff;
         int kmax = 0;
-        for (int i = tid; i < n_edges; i += 1024) {
+        for (int i = tid; i < n_edges; i += NT) {
             unsigned p = keys[i] >> KEY_POS_BITS;
             kmax = max(kmax, i - lower_bound_hi(keys, n_edges, p) + 1);
         }
@@ -530,9 +532,9 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
             else { a.meta[b].Kout = K; a.meta[b].errB = kerr; }
         }
         if (kerr) return;
-        for (int i = tid; i < K * SP; i += 1024) ell[i] = make_uint2(NO_STATE, 0u);
+        for (int i = tid; i < K * SP; i += NT) ell[i] = make_uint2(NO_STATE, 0u);
         __syncthreads();
-        for (int i = tid; i < n_edges; i += 1024) {
+        for (int i = tid; i < n_edges; i += NT) {
             unsigned p = keys[i] >> KEY_POS_BITS;
             int k = i - lower_bound_hi(keys, n_edges, p);
             int e = edge_at((int)(keys[i] & POS_MASK));
@@ -543,16 +545,16 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
     } else {
         // combine order: edges sorted by slot; CSR begin per slot; list of distinct emission ids
         uint4* crec = a.crec + edge_begin;
-        for (int i = tid; i < n_edges; i += 1024) {
+        for (int i = tid; i < n_edges; i += NT) {
             int e = edge_at((int)(keys[i] & POS_MASK));
             unsigned f = (unsigned)e_from[e] - smin, t = (unsigned)e_to[e] - smin;
             crec[i] = make_uint4(f | (t << 16), __float_as_uint(a.weights[e] * LOG2E), keys[i] >> KEY_POS_BITS, 0u);
         }
         int* cb = a.cbegin + goff;
-        for (int d = tid; d <= D; d += 1024) cb[d] = d == D ? n_edges : lower_bound_hi(keys, n_edges, (unsigned)d);
+        for (int d = tid; d <= D; d += NT) cb[d] = d == D ? n_edges : lower_bound_hi(keys, n_edges, (unsigned)d);
         int* de = a.demis + goff;
         const int nwords = (a.F + 31) >> 5;
-        for (int w = tid; w < nwords; w += 1024) {
+        for (int w = tid; w < nwords; w += NT) {
             unsigned bits = bitmap[w];
             int r = wordpfx[w];
             while (bits) {
@@ -561,7 +563,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
                 bits &= bits - 1;
             }
         }
-        for (int d = D + tid; d < DP; d += 1024) de[d] = 0;
+        for (int d = D + tid; d < DP; d += NT) de[d] = 0;
 
         // Frames in which a slot can carry probability mass.  An edge u->v is dead at frame t if
         // u cannot be reached from the start state in t edges or the end state cannot be reached
@@ -570,7 +572,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         // slot is dead there, so the result is the same, the states involved drop out of the
         // renormalisation, and for chain-like automata about half of the gather disappears.
         int dmax = 0, dmin = 0;
-        for (int i = tid; i < n_edges; i += 1024) {
+        for (int i = tid; i < n_edges; i += NT) {
             const int e = edge_at(i);
             const int df = (int)((unsigned)e_to[e] - (unsigned)e_from[e]);
             dmax = max(dmax, df); dmin = min(dmin, df);
@@ -582,15 +584,15 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         const int s_loc = (int)(st_state - smin), e_loc = (int)(en_state - smin);
         // one thread per edge; the per-slot minimum / maximum is taken with LDS atomics in the
         // memory of the sort keys, which are not needed any more once each thread has read its own
-        constexpr int EPT = EB_MAX / 1024;
+        constexpr int EPT = EB_MAX / NT;
         unsigned mykey[EPT];
 #pragma unroll
-        for (int j = 0; j < EPT; j++) mykey[j] = tid + j * 1024 < n_edges ? keys[tid + j * 1024] : ~0u;
+        for (int j = 0; j < EPT; j++) mykey[j] = tid + j * NT < n_edges ? keys[tid + j * NT] : ~0u;
         __syncthreads();
         int* s_tlo = (int*)keys;
         int* s_thi = (int*)keys + D_MAX;
         static_assert(2 * D_MAX <= EB_MAX, "band arrays reuse the key array");
-        for (int d = tid; d < DP; d += 1024) { s_tlo[d] = d < D ? (1 << 30) : 1; s_thi[d] = d < D ? -1 : 0; }
+        for (int d = tid; d < DP; d += NT) { s_tlo[d] = d < D ? (1 << 30) : 1; s_thi[d] = d < D ? -1 : 0; }
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
@@ -606,12 +608,14 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a) {
         __syncthreads();
         int2* tb = a.tband + goff;
         // (the best-path search reads every frame: values outside the band would have to be -inf there)
-        for (int d = tid; d < DP; d += 1024) tb[d] = (a.best_path || a.no_band) ? make_int2(0, 1 << 30) : make_int2(s_tlo[d], s_thi[d]);
+        for (int d = tid; d < DP; d += NT) tb[d] = (a.best_path || a.no_band) ? make_int2(0, 1 << 30) : make_int2(s_tlo[d], s_thi[d]);
     }
 }
 
-__global__ __launch_bounds__(1024) void fbw_prepare(PrepArgs a) {
-    prepare_sequence(a);      // every exit from it is taken by the whole workgroup
+template <int NT>
+__global__ __launch_bounds__(NT) void fbw_prepare(PrepArgs a) {
+    extern __shared__ unsigned prep_lds[];
+    prepare_sequence<NT>(a, prep_lds);      // every exit from it is taken by the whole workgroup
     // The recursion kernel of the overlapped schedule is already on the machine and waits for this
     // count: write this workgroup's tables back from the L2 of its XCD before it is raised.
     __syncthreads();
@@ -841,8 +845,13 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
             ew[j][k] = __uint_as_float(r.y);
         }
     }
+    if (tid < THREADS / 64) wmin[tid] = INF_F;
     RecCursor cur;
     recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
+    // Waves without a state leave: they would only compete with the others for issue slots on
+    // their SIMD, and a barrier counts the waves that are still there.  Their entries of wmin keep
+    // the +inf written above.
+    if (J == 1 && (tid & ~63) >= SP) return;
     for (int i = 0; i < cur.nsteps; i += 2) {
         recurse_step<SYNC, THREADS, J, KT, ST>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
         if (i + 1 < cur.nsteps)
@@ -1485,6 +1494,17 @@ struct Pipeline {
 Pipeline g_pipe[MAX_DEVICES];
 std::mutex g_mutex;
 
+// LDS of a preparation workgroup: sort keys, emission bitmap and its prefix counts
+size_t prep_lds_bytes(int F) { return (size_t)EB_MAX * 4 + (F <= F_BITMAP_MAX ? (size_t)((F + 31) >> 5) * 8 : 0); }
+
+// 1024-thread workgroups sort fastest, but only two of them fit on a compute unit: batches that
+// would need a second round of them take 512-thread workgroups, four to a unit.
+void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
+    const size_t lds = prep_lds_bytes(pa.F);
+    if (3 * pa.B > 2 * P.n_cu) hipLaunchKernelGGL(fbw_prepare<512>, dim3(3, pa.B), dim3(512), lds, s, pa);
+    else hipLaunchKernelGGL(fbw_prepare<1024>, dim3(3, pa.B), dim3(1024), lds, s, pa);
+}
+
 int pipeline_init(Pipeline& p) {
     if (p.ready) return I6FBW_OK;
     int dev = 0;
@@ -1497,6 +1517,8 @@ int pipeline_init(Pipeline& p) {
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
         HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     p.ready = true;
@@ -1697,7 +1719,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     }
     {
         StageTimer tm(0, s);
-        hipLaunchKernelGGL(fbw_prepare, dim3(3, B), dim3(1024), 0, s, pa);
+        launch_prepare(P, pa, s);
         HIP_TRY(hipGetLastError());
     }
     if (overlap && !early) {
