@@ -155,3 +155,20 @@ def test_fast_path_at_capacity(oracle):
     assert W.n_states == 4096 and W.E == 8190
     W.seq_lens[:] = W.T
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=1)
+
+
+@pytest.mark.parametrize("shuffle", [False, True], ids=["grouped", "shuffled"])
+def test_many_short_sequences(oracle, shuffle):
+    """More sequences than two large preparation workgroups per compute unit can take in one round: the
+    preparation runs with smaller workgroups; edge list grouped by sequence and in random order."""
+    W = make_workload("ctc", T=40, B=300, F=400, shuffle_edges=shuffle)
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
+
+
+@pytest.mark.parametrize("n_labels", [60, 450, 1200], ids=["small", "over-1024-edges", "over-512-classes"])
+def test_one_class_on_many_edges(oracle, n_labels):
+    """CTC automata put the blank class on every other state: its posterior is a sum over hundreds or
+    thousands of edges per frame, which the dense write takes with a whole wave (both of its paths: edges
+    in registers, edges staged in passes)."""
+    W = make_workload("ctc", T=3 * n_labels, B=2, F=n_labels + 200, n_labels=(n_labels, n_labels + 1))
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
