@@ -95,6 +95,9 @@ __host__ __device__ inline long long round16(long long x) { return (x + 15) & ~1
 // prefix sum over sequences (and no cross-workgroup dependency) is needed.
 __host__ __device__ inline long long state_off(long long edge_begin, int b) { return round16(2 * edge_begin) + 32LL * b; }
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
+// Entries of a sequence's renumbering table (see local_state) and the home position of a state id in it
+__device__ __forceinline__ unsigned renum_capacity(int n_edges) { return (unsigned)KMAX * (2u * (unsigned)n_edges + 16u); }
+__device__ __forceinline__ unsigned renum_home(int id, unsigned cap) { return __umulhi((unsigned)id * 2654435761u, cap); }
 
 struct Layout {
     size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, offA, offB, alpha, beta, gtab, total;
@@ -321,7 +324,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     unsigned* bitmap = lds + EB_MAX;
     int* wordpfx = (int*)(bitmap + ((a.F + 31) >> 5));
     __shared__ int wsum[NT / 64];
-    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin;
+    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin, s_count;
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -331,7 +334,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int32_t* e_seq = a.edges + 3 * a.edge_stride;
     const int E = a.E;
 
-    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; }
+    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; s_count = 0; }
     __syncthreads();
     const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
     int unsorted = 0;
@@ -392,11 +395,15 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // lengths beyond T are read as T
     const int L = a.best_path ? ((int)sl < 0 ? 0 : min((int)sl, a.T)) : ((sl >= 1u && sl <= (unsigned)a.T) ? (int)sl : 0);
     long long S = (long long)smax - smin + 1;
-    if (!err && n_edges > 0 && S > 2LL * n_edges + 2) err = I6FBW_ERR_SEQ_SPARSE_STATES;
+    // ids spread over a range much larger than their number (the workspace is sized by the edge
+    // count): the states get dense numbers (below), and the sequence takes the general path, which
+    // looks them up
+    const bool sparse = !err && n_edges > 0 && S > 2LL * n_edges + 2;
+    if (sparse) generic = 1;
     if (n_edges == 0) S = 1;
     if (!err && S > S_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
     if (!err && a.force_generic && n_edges > 0) generic = 1;
-    const int SP = (int)round16(S);
+    int SP = (int)round16(S);
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
     // i-th edge of this sequence in input order
@@ -430,6 +437,48 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
+    int start_loc = (int)(st_state - smin), end_loc = (int)(en_state - smin);
+    if (sparse && role == 2) {
+        // Dense numbers for the states, in the order in which they are entered into the table that
+        // local_state() reads (any numbering will do: the general path never compares ids, and the
+        // distance bounds of min_steps hold for every numbering).
+        int2* tab = (int2*)a.ellA + (size_t)KMAX * soff;
+        const unsigned cap = renum_capacity(n_edges);
+        for (unsigned i = tid; i < cap; i += NT) { store_agent(&tab[i].x, 0); store_agent(&tab[i].y, 0); }
+        wait_stores();
+        __syncthreads();        // also: the edge list written above
+        auto enter = [&](const int id) {
+            unsigned h = renum_home(id, cap);
+            while (true) {
+                const int seen = atomicCAS(&tab[h].x, 0, id + 1);
+                if (seen == 0) { store_agent(&tab[h].y, atomicAdd(&s_count, 1)); return; }
+                if (seen == id + 1) return;
+                h = h + 1 == cap ? 0 : h + 1;
+            }
+        };
+        auto number_of = [&](const int id) -> int {
+            unsigned h = renum_home(id, cap);
+            while (true) {
+                const int key = load_agent(&tab[h].x);
+                if (key == id + 1) return load_agent(&tab[h].y);
+                if (key == 0) return 0;
+                h = h + 1 == cap ? 0 : h + 1;
+            }
+        };
+        for (int i = tid; i < n_edges; i += NT) {
+            const int e = edge_at(i);
+            enter(e_from[e]);
+            enter(e_to[e]);
+        }
+        if (tid == 0) { enter((int)st_state); enter((int)en_state); }
+        wait_stores();
+        __syncthreads();
+        S = s_count;
+        SP = (int)round16(S);
+        start_loc = number_of((int)st_state);
+        end_loc = number_of((int)en_state);
+    }
+
     if (role == 2) {
         // hand-off area of this sequence: progress counters and gather flags start at zero
         const int nstrip = (a.T + TG - 1) / TG;
@@ -441,9 +490,10 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         SeqMeta* m = a.meta + b;
         m->edge_begin = edge_begin; m->n_edges = n_edges; m->state_min = (int)smin;
         m->S = (int)S; m->SP = SP; m->D = D; m->DP = DP; m->L = L;
-        m->start_local = (int)(st_state - smin); m->end_local = (int)(en_state - smin);
+        m->start_local = start_loc; m->end_local = end_loc;
         m->err = err ? err : (generic ? SEQ_GENERIC : 0);
-        m->pad = sorted ? 1 : 0;         // bit 0: the edges of the sequence are contiguous in the input
+        // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered
+        m->pad = (sorted ? 1 : 0) | (sparse ? 2 : 0);
     }
     if (err || generic || n_edges == 0) {
         if (tid == 0) {
@@ -1669,7 +1719,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.ascending = 0;
     GenArgs gen;
     gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
-    gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx;
+    gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx; gen.renum = (const int2*)pa.ellA;
     RecArgs ra;
     ra.gen = gen;
     ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab; ra.gtab_rw = ga.gtab;
@@ -1801,7 +1851,7 @@ const char* i6fbw_strerror(int code) {
         case I6FBW_ERR_LAUNCH: return "HIP call failed";
         case I6FBW_ERR_F_TOO_LARGE: return "number of emission classes F exceeds the supported maximum";
         case I6FBW_ERR_SEQ_TOO_MANY_EDGES: return "a sequence has more edges than supported (8192)";
-        case I6FBW_ERR_SEQ_SPARSE_STATES: return "state ids of a sequence span more than 2*edges+2 ids";
+        case I6FBW_ERR_SEQ_SPARSE_STATES: return "state ids of a sequence span more than 2*edges+2 ids (not reported any more)";
         case I6FBW_ERR_SEQ_DEGREE: return "a state has more than 8 incoming or outgoing edges";
         case I6FBW_ERR_SEQ_TOO_LARGE: return "a sequence has more than 4096 states or distinct emissions";
         case I6FBW_ERR_BAD_INDEX: return "sequence, emission or state index out of range";

@@ -83,3 +83,19 @@ def random_fsa(rng, B, F, max_states=4, max_edges=8, T=5):
 def posterior(out):
     """exp(-out): what FastBaumWelchLoss.backward returns (fbw/__init__.py:40-44)."""
     return np.exp(-out.astype(np.float64))
+
+
+def spread_state_ids(edges, start_end, n_states, how="permute", seed=5):
+    """The same automata under other state ids: "stride" multiplies every id by 11 (each sequence keeps a
+    range of its own, eleven times as wide), "permute" draws the ids at random from a range three times as
+    large (the ranges of all sequences overlap)."""
+    if how == "stride":
+        new_id = np.arange(n_states, dtype=np.int64) * 11 + 3
+        total = n_states * 11 + 3
+    else:
+        total = n_states * 3
+        new_id = np.random.default_rng(seed).permutation(total)[:n_states]
+    out = edges.copy()
+    out[0] = new_id[edges[0]]
+    out[1] = new_id[edges[1]]
+    return out, new_id[start_end].astype(np.int32), int(total)

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import spread_state_ids
 from tests.test_fbw_gpu import check_against_oracle, schedule  # noqa: F401  (autouse fixture: both schedules)
 
 pytestmark = pytest.mark.gpu
@@ -77,3 +78,38 @@ def test_status_is_clean_for_general_path():
     am = rng.uniform(0.1, 3.0, size=(12, 1, 9)).astype(np.float32)
     P = DeviceProblem(am, edges, weights, np.array([[s], [e]], np.int32), np.array([12], np.int32), n)
     P.run(cabi.OUT_PROB)                 # raises on any reported status
+
+
+@pytest.mark.parametrize("how", ["stride", "permute"])
+@pytest.mark.parametrize("name,kw", [("cart", dict(T=80, B=4, F=120)), ("ctc", dict(T=50, B=9, F=60, shuffle_edges=True)),
+                                     ("monophone", dict(T=400, B=2, F=70, n_labels=(90, 100)))])
+def test_widely_spread_state_ids(oracle, how, name, kw):
+    """The reference indexes its state buffers with the ids as they come, so ids need not be compact.
+    Sequences whose ids span much more than their number get dense numbers on the device (and take the
+    general path); the oracle sees the spread ids as they are."""
+    W = make_workload(name, **kw)
+    edges, start_end, n_states = spread_state_ids(W.edges, W.start_end_states, W.n_states, how)
+    out, loss = check_against_oracle(oracle, (W.am_scores, edges, W.weights, start_end, W.seq_lens, n_states), bitwise=False)
+    # and it is the result of the compact numbering
+    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    np.testing.assert_allclose(loss, want_loss, rtol=1e-5, atol=1e-6)
+
+
+def test_two_sequences_naming_the_same_states(oracle):
+    """Each sequence works on its own copy of the states it names, also when the ids are renumbered: two
+    sequences over the same widely spread ids do not disturb each other."""
+    W = make_workload("cart", T=40, B=1, F=50)
+    edges, start_end, n_states = spread_state_ids(W.edges, W.start_end_states, W.n_states, "stride")
+    twice = np.concatenate([edges, edges], axis=1)
+    twice[3, edges.shape[1]:] = 1
+    am = np.concatenate([W.am_scores, W.am_scores[::-1]], axis=1).copy()
+    args1 = (W.am_scores, edges, W.weights, start_end, W.seq_lens, n_states)
+    args2 = (am[:, 1:].copy(), edges, W.weights, start_end, W.seq_lens, n_states)
+    from tests.gpu_util import run_cabi
+    from i6_native_ops_amd import cabi
+    post, loss = run_cabi(am, twice, np.concatenate([W.weights, W.weights]), np.concatenate([start_end, start_end], axis=1),
+                          np.concatenate([W.seq_lens, W.seq_lens]), n_states, out_mode=cabi.OUT_PROB)
+    for b, args in enumerate((args1, args2)):
+        want_out, want_loss = oracle.fbw_oracle(*args)
+        np.testing.assert_allclose(loss[:, b], want_loss[:, 0], rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(post[:, b], np.exp(-want_out[:, 0].astype(np.float64)), rtol=0, atol=1e-4)

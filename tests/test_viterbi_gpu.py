@@ -8,6 +8,7 @@ import torch
 
 from i6_native_ops_amd import cabi
 from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import spread_state_ids
 from tests.helpers import random_fsa
 from tests.test_oracle_viterbi import viterbi_fixture
 
@@ -121,13 +122,24 @@ def test_size_classes(oracle, kind):
 
 
 def test_device_status():
-    """State ids spread over far more ids than the sequence has edges are reported; the sequence gets
-    score NaN and an all-zero alignment."""
-    edges = np.array([[0, 50, 1, 0], [50, 50, 2, 0]], dtype=np.int32).T.copy()
+    """An index out of range is reported; the sequence gets score NaN and an all-zero alignment."""
+    edges = np.array([[0, 1, 1, 0], [1, 1, 9, 0]], dtype=np.int32).T.copy()      # emission class 9 of 4
     am = np.zeros((2, 1, 4), dtype=np.float32)
-    a, s, code = run_cabi_viterbi(am, edges, np.zeros(2, np.float32), np.array([[0], [50]], np.int32),
-                                  np.array([2], np.int32), 51, check=False)
-    assert code == -11 and np.isnan(s[0]) and (a == 0).all()
+    a, s, code = run_cabi_viterbi(am, edges, np.zeros(2, np.float32), np.array([[0], [1]], np.int32),
+                                  np.array([2], np.int32), 2, check=False)
+    assert code == -14 and np.isnan(s[0]) and (a == 0).all()
+
+
+@pytest.mark.parametrize("how", ["stride", "permute"])
+def test_widely_spread_state_ids(oracle, how):
+    """State ids of a sequence far apart get dense numbers on the device; the result is that of the same
+    automata with compact ids, bit for bit."""
+    wl = make_workload("cart", T=60, B=5, F=90)
+    am, w = -wl.am_scores, -wl.weights
+    want = oracle.viterbi_oracle(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states)
+    edges, start_end, n_states = spread_state_ids(wl.edges, wl.start_end_states, wl.n_states, how)
+    assert_identical(run_cabi_viterbi(am, edges, w, start_end, wl.seq_lens, n_states)[:2], want)
+    assert_identical(oracle.viterbi_oracle(am, edges, w, start_end, wl.seq_lens, n_states), want)
 
 
 @pytest.mark.parametrize("kind", ["degree", "many_states", "many_classes", "ties"])

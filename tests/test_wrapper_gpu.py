@@ -110,13 +110,13 @@ def test_device_side_status_is_reported():
     bad[3, 0] = 3                       # sequence index >= B
     with pytest.raises(RuntimeError, match="index out of range"):
         core.fbw(am, bad, weights, se, seq_lens, n)
-    # state ids of one sequence spread over far more ids than it has edges
+    # state ids of one sequence spread over far more ids than it has edges: renumbered, same result
+    want_out, want_loss = core.fbw(am, edges, weights, se, seq_lens, n)
     sparse = edges.clone()
-    sparse[1, 1] = 40
-    sparse[0, 2] = 40
-    sparse[1, 2] = 40
-    with pytest.raises(RuntimeError, match="span more than"):
-        core.fbw(am, sparse, weights, torch.tensor([[0], [40]], dtype=torch.int32, device="cuda"), seq_lens, 41)
+    sparse[:2][edges[:2] == se[1, 0]] = 40
+    out, loss = core.fbw(am, sparse, weights, torch.tensor([[int(se[0, 0])], [40]], dtype=torch.int32, device="cuda"), seq_lens, 41)
+    torch.testing.assert_close(loss, want_loss, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(torch.exp(-out), torch.exp(-want_out), rtol=0, atol=1e-5)
     # a state with 9 incoming edges is beyond the fast kernels, not beyond the library
     many = torch.tensor([[0] * 9, [1] * 9, [0] * 9, [0] * 9], dtype=torch.int32, device="cuda")
     out, loss = core.fbw(am, many, torch.zeros(9, device="cuda"), se, torch.tensor([1], dtype=torch.int32, device="cuda"), n)
