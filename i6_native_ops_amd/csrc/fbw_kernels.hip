@@ -1064,17 +1064,17 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
     const int K = dir ? m.Kout : m.Kin;
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
-    // (Fewer specialisations for double: it is the rare case.)
+    // (No six-edge specialisation for double: it is the rare case.)
     constexpr bool F32 = sizeof(ST) == 4;
     if (cls == 1) {
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
-        else if (F32 && K <= 3) recurse_compute<SYNC, T_, 1, F32 ? 3 : 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (K <= 3) recurse_compute<SYNC, T_, 1, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (F32 && K <= 6) recurse_compute<SYNC, T_, 1, F32 ? 6 : KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute<SYNC, T_, 1, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
     } else if (cls == 2) {
         if (K <= 2) recurse_compute<SYNC, T_, 4, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
-        else if (F32 && K <= 3) recurse_compute<SYNC, T_, 4, F32 ? 3 : 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (K <= 3) recurse_compute<SYNC, T_, 4, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 4, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, 4 * T_);
     } else {
