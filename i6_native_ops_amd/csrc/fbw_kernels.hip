@@ -40,6 +40,8 @@
 namespace {
 
 constexpr int KMAX = 8;               // in-/out-degree held in registers by the recursion
+constexpr int KWIDE = 15;             // largest degree the edge tables hold (re-read from memory per frame beyond KMAX);
+                                      // the best-path search packs the edge's rank into four bits, with 15 | 4095 << 0 reserved
 constexpr int EB_MAX = 8192;          // edges of one sequence (capacity of the LDS sort)
 constexpr int F_BITMAP_MAX = 131072;  // emission ids covered by the LDS presence bitmap
 constexpr int S_MAX = 4096;           // states of one sequence
@@ -576,7 +578,13 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         if (kmax) atomicMax(&s_kmax, kmax);
         __syncthreads();
         const int K = s_kmax;
-        const int kerr = K > KMAX ? (gen_ok ? SEQ_GENERIC : I6FBW_ERR_SEQ_DEGREE) : 0;
+        // Up to KMAX edges per state fit every sequence's share of the table area (KMAX entries per
+        // state).  A larger degree, up to KWIDE, is taken as long as the table still fits the share
+        // -- it does unless most states have few edges; the recursion then re-reads the table each
+        // frame.  Beyond that: general path.
+        const long long share = state_off((long long)edge_begin + n_edges, b + 1) - soff;
+        const bool fits = K <= KMAX || (K <= KWIDE && (long long)K * SP <= (long long)KMAX * share);
+        const int kerr = fits ? 0 : (gen_ok ? SEQ_GENERIC : I6FBW_ERR_SEQ_DEGREE);
         if (tid == 0) {
             if (role == 0) { a.meta[b].Kin = K; a.meta[b].errA = kerr; }
             else { a.meta[b].Kout = K; a.meta[b].errB = kerr; }
@@ -936,6 +944,24 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
             cur.c += (double)pend;
         }
         float rmin = INF_F;
+        if (K > KMAX) {
+            // degree beyond the unrolled body: two passes over the state's table column
+            for (int s = tid; s < SP; s += THREADS) {
+                auto value = [&](int k) -> ST {
+                    const uint2 r = ell[(size_t)k * SP + s];
+                    const unsigned other = r.x & 0xFFFFu;
+                    return other == NO_STATE ? (ST)INF_F : stc[other] + (ST)(__uint_as_float(r.y) + amc[r.x >> 16]);
+                };
+                ST mn = (ST)INF_F;
+                for (int k = 0; k < K; k++) mn = state_min(mn, value(k));
+                float sum = 0.f;
+                for (int k = 0; k < K; k++) sum += __builtin_amdgcn_exp2f((float)(mn - value(k)));
+                const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
+                stn[s] = r;
+                store_x<SYNC>(cur.wp + s, (float)r);
+                rmin = fminf(rmin, (float)r);
+            }
+        } else
         for (int s = tid; s < SP; s += THREADS) {
             ST v[KMAX];
             ST mn = (ST)INF_F;
@@ -1066,7 +1092,9 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     // (No six-edge specialisation for double: it is the rare case.)
     constexpr bool F32 = sizeof(ST) == 4;
-    if (cls == 1) {
+    if (K > KMAX) {
+        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
+    } else if (cls == 1) {
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);

@@ -1,4 +1,4 @@
-"""Automata beyond the capacity of the fast kernels (more than 8 edges into or out of a state,
+"""Automata beyond the capacity of the fast kernels (more than 15 edges into or out of a state,
 more than 8192 edges, 4096 states or 4096 distinct emissions in one sequence, more emission
 classes than the LDS row image holds) take the general path inside the same kernels.  Same parity
 bar as everything else, under both schedules, also mixed with ordinary sequences in one batch."""
@@ -113,3 +113,25 @@ def test_two_sequences_naming_the_same_states(oracle):
         want_out, want_loss = oracle.fbw_oracle(*args)
         np.testing.assert_allclose(loss[:, b], want_loss[:, 0], rtol=1e-5, atol=1e-6)
         np.testing.assert_allclose(post[:, b], np.exp(-want_out[:, 0].astype(np.float64)), rtol=0, atol=1e-4)
+
+
+@pytest.mark.parametrize("n_mid", [9, 12, 15, 16])
+def test_degree_just_beyond_the_register_tables(oracle, n_mid):
+    """Degrees 9 to 15 still run on the table-driven kernels (the table is re-read from memory each frame;
+    fixed summation order, so the result is reproducible bit for bit); 16 and more take the general path.
+    A hub of that degree inside an ordinary left-to-right automaton, and the bare fan."""
+    rng = np.random.default_rng(100 + n_mid)
+    W = make_workload("cart", T=90, B=3, F=80, n_labels=(8, 12))
+    edges, weights = W.edges.copy(), W.weights.copy()
+    for b in range(W.B):                                     # n_mid extra edges into the end state, out of the start state
+        states = np.unique(edges[:2, edges[3] == b])
+        s, e = int(W.start_end_states[0, b]), int(W.start_end_states[1, b])
+        frm = rng.choice(states, size=n_mid); to = rng.choice(states, size=n_mid)
+        extra = np.array([np.concatenate([frm, [s] * n_mid]), np.concatenate([[e] * n_mid, to]),
+                          rng.integers(0, W.F, size=2 * n_mid), [b] * (2 * n_mid)], dtype=np.int32)
+        edges = np.concatenate([edges, extra], axis=1)
+        weights = np.concatenate([weights, rng.uniform(0.2, 2.0, size=2 * n_mid).astype(np.float32)])
+    check_against_oracle(oracle, (W.am_scores, edges, weights, W.start_end_states, W.seq_lens, W.n_states), bitwise=n_mid <= 15 - 3)
+    e2, w2, s2, t2, n2 = fan(rng, 12, 9, n_mid)
+    am = rng.uniform(0.1, 3.0, size=(12, 1, 9)).astype(np.float32)
+    check_against_oracle(oracle, (am, e2, w2, np.array([[s2], [t2]], np.int32), np.array([12], np.int32), n2), bitwise=n_mid <= 15)

@@ -142,13 +142,13 @@ def test_widely_spread_state_ids(oracle, how):
     assert_identical(oracle.viterbi_oracle(am, edges, w, start_end, wl.seq_lens, n_states), want)
 
 
-@pytest.mark.parametrize("kind", ["degree", "many_states", "many_classes", "ties"])
+@pytest.mark.parametrize("kind", ["degree", "degree12", "ties12", "many_states", "many_classes", "ties"])
 def test_general_path(oracle, kind):
-    """Beyond the capacity of the fast kernels (more than 8 edges into a state, more than 4096 states,
+    """Beyond the capacity of the fast kernels (more than 15 edges into a state (9 to 15: tables re-read per frame), more than 4096 states,
     more emission classes than the bitmap holds): same bits as the oracle, ties included."""
     rng = np.random.default_rng(77)
-    if kind in ("degree", "ties"):
-        T, F, n_mid = 14, 9, 25
+    if kind in ("degree", "ties", "degree12", "ties12"):        # degree 12: tables re-read per frame; 25: general path
+        T, F, n_mid = 14, 9, (12 if kind.endswith("12") else 25)
         frm, to, emis = [], [], []
         for i in range(n_mid):
             frm += [0, 1 + i, 1 + i]
@@ -157,7 +157,7 @@ def test_general_path(oracle, kind):
         edges = np.array([frm, to, emis, [0] * len(frm)], dtype=np.int32)
         weights = rng.uniform(-1.5, 0.0, size=len(frm)).astype(np.float32)
         am = -rng.uniform(0.1, 3.0, size=(T, 1, F)).astype(np.float32)
-        if kind == "ties":
+        if kind.startswith("ties"):
             weights[:] = -0.5
             am = np.round(am)
         args = (am, edges, weights, np.array([[0], [n_mid + 1]], np.int32), np.array([11], np.int32), n_mid + 2)
