@@ -193,3 +193,48 @@ def test_graph_capture_of_a_large_call(oracle):
         torch.cuda.synchronize()
         assert torch.equal(P.loss, eager_loss)
         assert torch.equal(P.out, eager_post)
+
+
+@pytest.mark.parametrize("overlap", [-1, 1], ids=["automatic", "overlapped"])
+def test_two_host_threads_on_their_own_streams(overlap):
+    """Two threads call the library at the same time, each on its own stream and workspace (the
+    library's streams and events are shared by all callers of a device): every call gives the result
+    of the same call made alone, bit for bit."""
+    import threading
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import DeviceProblem
+    workloads = [make_workload("cart", T=400, B=16, F=12001), make_workload("ctc", T=100, B=40, F=300)]
+    problems = [DeviceProblem(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states) for W in workloads]
+    cabi.set_overlap(overlap)
+    try:
+        want = []
+        for P in problems:
+            post, loss = P.run(cabi.OUT_PROB)
+            torch.cuda.synchronize()
+            want.append((post.clone(), loss.clone()))
+        failures = []
+
+        def work(i):
+            try:
+                P = problems[i]
+                stream = torch.cuda.Stream()
+                with torch.cuda.stream(stream):
+                    for it in range(12):
+                        P.loss.fill_(-1.0)
+                        post, loss = P.run(cabi.OUT_PROB)
+                        stream.synchronize()
+                        if not torch.equal(loss, want[i][1]):
+                            failures.append((i, it, "loss"))
+                    if not torch.equal(post, want[i][0]):
+                        failures.append((i, "posteriors"))
+            except Exception as exc:        # noqa: BLE001  (reported below, in the main thread)
+                failures.append((i, repr(exc)))
+
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not failures, failures
+    finally:
+        cabi.set_overlap(-1)
