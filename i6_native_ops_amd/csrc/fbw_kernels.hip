@@ -389,9 +389,8 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     if (s_bad || st_state >= (unsigned)a.n_states || en_state >= (unsigned)a.n_states) err = I6FBW_ERR_BAD_INDEX;
     // Sequences beyond the capacity of the fast kernels take the general path (generic_path.inc,
     // generic_viterbi).
-    constexpr bool gen_ok = true;
     int generic = 0;
-    if (!err && n_edges > EB_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_MANY_EDGES; }
+    if (!err && n_edges > EB_MAX) generic = 1;
     const unsigned sl = (unsigned)a.seq_lens[b];
     // full sum: a length outside [1, T] leaves the sequence without probability mass; best path:
     // lengths beyond T are read as T
@@ -403,7 +402,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const bool sparse = !err && n_edges > 0 && S > 2LL * n_edges + 2;
     if (sparse) generic = 1;
     if (n_edges == 0) S = 1;
-    if (!err && S > S_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
+    if (!err && S > S_MAX) generic = 1;
     if (!err && a.force_generic && n_edges > 0) generic = 1;
     int SP = (int)round16(S);
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
@@ -435,7 +434,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         int run = block_excl_scan(c, wsum, NT / 64, &D);
         for (int w = w0; w < w1; w++) { wordpfx[w] = run; run += __popc(bitmap[w]); }
         __syncthreads();
-        if (D > D_MAX) { if (gen_ok) generic = 1; else err = I6FBW_ERR_SEQ_TOO_LARGE; }
+        if (D > D_MAX) generic = 1;
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
@@ -584,7 +583,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         // frame.  Beyond that: general path.
         const long long share = state_off((long long)edge_begin + n_edges, b + 1) - soff;
         const bool fits = K <= KMAX || (K <= KWIDE && (long long)K * SP <= (long long)KMAX * share);
-        const int kerr = fits ? 0 : (gen_ok ? SEQ_GENERIC : I6FBW_ERR_SEQ_DEGREE);
+        const int kerr = fits ? 0 : SEQ_GENERIC;
         if (tid == 0) {
             if (role == 0) { a.meta[b].Kin = K; a.meta[b].errA = kerr; }
             else { a.meta[b].Kout = K; a.meta[b].errB = kerr; }
@@ -1593,7 +1592,7 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
     for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
-        HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
@@ -1717,7 +1716,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     const int forced = g_overlap_mode;
     // By default only where it pays: a large dense tensor, and a batch whose recursion workgroups
     // leave wave slots free on every compute unit (with two of them on each unit the gather crawls:
-    // T=200, B=256, F=5001 takes 0.59 ms overlapped against 0.48 ms stage after stage).
+    // T=200, B=256, F=5001 takes 0.49 ms overlapped against 0.40 ms stage after stage).
     bool overlap = forced >= 0 ? forced != 0 : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu);
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
@@ -1784,7 +1783,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     };
     if (overlap) {
         // The library streams are released when the scan is done, i.e. while the preparation's
-        // workgroups are being placed.  The recursion's 2B large workgroups need ten free wave
+        // workgroups are being placed.  The recursion's 2B large workgroups need nine free wave
         // slots on one compute unit each and find them while the machine is still almost empty;
         // they wait in memory for the preparation to finish (fbw_prepare counts its workgroups),
         // and their loader waves later for the gather's strip flags.
