@@ -98,11 +98,11 @@ __host__ __device__ inline long long round16(long long x) { return (x + 15) & ~1
 __host__ __device__ inline long long state_off(long long edge_begin, int b) { return round16(2 * edge_begin) + 32LL * b; }
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 // Entries of a sequence's renumbering table (see local_state) and the home position of a state id in it
-__device__ __forceinline__ unsigned renum_capacity(int n_edges) { return (unsigned)KMAX * (2u * (unsigned)n_edges + 16u); }
+__device__ __forceinline__ unsigned renum_capacity(int n_edges) { return 2u * (2u * (unsigned)n_edges + 16u); }
 __device__ __forceinline__ unsigned renum_home(int id, unsigned cap) { return __umulhi((unsigned)id * 2654435761u, cap); }
 
 struct Layout {
-    size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, renum, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
 };
 
@@ -124,6 +124,7 @@ Layout make_layout(long long T, long long B, long long E) {
     l.cbegin = o;   o = align256(o + sizeof(int) * l.gg_total);
     l.demis = o;    o = align256(o + sizeof(int) * l.gg_total);
     l.tband = o;    o = align256(o + sizeof(int2) * l.gg_total);
+    l.renum = o;    o = align256(o + sizeof(int2) * 2 * l.ss_total);
     l.offA = o;     o = align256(o + sizeof(double) * B * T);
     l.offB = o;     o = align256(o + sizeof(double) * B * T);
     l.alpha = o;    o = align256(o + sizeof(float) * l.ss_total * T);
@@ -241,6 +242,7 @@ struct PrepArgs {
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
     int force_generic;  // F is too large for the emission bitmap or the row image: every sequence takes the general path
+    int2* renum;        // renumbering tables, two entries per state of room (see local_state)
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
 
@@ -291,6 +293,23 @@ __device__ inline int block_excl_scan(int v, int* wsum, int nwaves, int* total) 
     __syncthreads();
     *total = tot;
     return base + incl - v;
+}
+
+// In-place bitonic sort of N (a power of two) keys in LDS by the whole workgroup.
+template <int NT>
+__device__ inline void lds_bitonic_sort(unsigned* keys, const int N) {
+    for (int k = 2; k <= N; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = threadIdx.x; i < N; i += NT) {
+                const int ixj = i ^ j;
+                if (ixj > i) {
+                    const unsigned x = keys[i], y = keys[ixj];
+                    if ((x > y) == ((i & k) == 0)) { keys[i] = y; keys[ixj] = x; }
+                }
+            }
+            __syncthreads();
+        }
+    }
 }
 
 constexpr int KEY_POS_BITS = 13;   // EB_MAX = 2^13 positions; the primary key sits above them
@@ -400,11 +419,15 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // count): the states get dense numbers (below), and the sequence takes the general path, which
     // looks them up
     const bool sparse = !err && n_edges > 0 && S > 2LL * n_edges + 2;
-    if (sparse) generic = 1;
+    // up to this many edges the renumbering is done in LDS, the same way by all three roles, and the
+    // sequence stays on the fast kernels: the 2n+2 ids fit the key array, and afterwards the n edge
+    // keys its lower half and the distinct ids its upper half
+    constexpr int RENUM_LDS_EDGES = EB_MAX / 2 - 1;
+    bool ranked = sparse && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
+    if (sparse && !ranked) generic = 1;
     if (n_edges == 0) S = 1;
-    if (!err && S > S_MAX) generic = 1;
+    if (!err && !sparse && S > S_MAX) generic = 1;
     if (!err && a.force_generic && n_edges > 0) generic = 1;
-    int SP = (int)round16(S);
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
     // i-th edge of this sequence in input order
@@ -417,6 +440,55 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         for (int i = lo; i < hi; i++)
             if ((unsigned)e_seq[i] == (unsigned)b) eidx[pos++] = i;
     }
+    // Widely spread ids, in LDS: all ids the sequence names are sorted, the distinct ones are kept in
+    // ascending order in the upper half of the key array, and a state's number is its rank there
+    // (binary search).  Every role arrives at the same numbers.
+    unsigned* uniq = keys + EB_MAX / 2;
+    if (ranked) {
+        __syncthreads();        // the edge list written above
+        const int M = 2 * n_edges + 2;
+        int N2 = 2;
+        while (N2 < M) N2 <<= 1;
+        for (int i = tid; i < N2; i += NT) {
+            unsigned k = ~0u;
+            if (i < 2 * n_edges) { const int e = edge_at(i >> 1); k = (unsigned)((i & 1) ? e_to[e] : e_from[e]); }
+            else if (i == 2 * n_edges) k = st_state;
+            else if (i == 2 * n_edges + 1) k = en_state;
+            keys[i] = k;
+        }
+        __syncthreads();
+        lds_bitonic_sort<NT>(keys, N2);
+        constexpr int CH = EB_MAX / NT;
+        unsigned mine[CH];
+        int cnt = 0;
+#pragma unroll
+        for (int j = 0; j < CH; j++) {
+            const int i = tid * CH + j;
+            mine[j] = ~0u;
+            if (i < M && (i == 0 || keys[i - 1] != keys[i])) { mine[j] = keys[i]; cnt++; }
+        }
+        int total;
+        int at = block_excl_scan(cnt, wsum, NT / 64, &total);       // its barriers come after every read above
+        S = total;
+        if (total > S_MAX) { ranked = false; generic = 1; }          // too many states for the fast kernels (and for the upper half)
+        else {
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                if (mine[j] != ~0u) uniq[at++] = mine[j];
+        }
+        __syncthreads();
+    }
+    // state id -> number within the sequence
+    auto local = [&](const unsigned id) -> unsigned {
+        if (!ranked) return id - smin;
+        int lo_ = 0, hi_ = (int)S;
+        while (lo_ < hi_) {
+            const int mid = (lo_ + hi_) >> 1;
+            if (uniq[mid] < id) lo_ = mid + 1; else hi_ = mid;
+        }
+        return (unsigned)lo_;
+    };
+    int SP = (int)round16(S);
     if (!err && !generic && n_edges > 0) {
         // emission presence bitmap -> slot = rank of the emission id among the distinct ones
         const int nwords = (a.F + 31) >> 5;
@@ -438,12 +510,14 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
-    int start_loc = (int)(st_state - smin), end_loc = (int)(en_state - smin);
+    int start_loc = (int)local(st_state), end_loc = (int)local(en_state);
     if (sparse && role == 2) {
-        // Dense numbers for the states, in the order in which they are entered into the table that
-        // local_state() reads (any numbering will do: the general path never compares ids, and the
-        // distance bounds of min_steps hold for every numbering).
-        int2* tab = (int2*)a.ellA + (size_t)KMAX * soff;
+        // The general path looks the numbers up in an open-addressing table {id + 1, number} (see
+        // local_state), which is written for every sequence with spread ids: the other two roles may
+        // still send it there.  Numbers: the ranks from above, or, for a sequence too large for
+        // that, the order in which the ids happen to be entered (any numbering will do: the general
+        // path never compares ids, and the distance bounds of min_steps hold for every numbering).
+        int2* tab = a.renum + 2 * soff;
         const unsigned cap = renum_capacity(n_edges);
         for (unsigned i = tid; i < cap; i += NT) { store_agent(&tab[i].x, 0); store_agent(&tab[i].y, 0); }
         wait_stores();
@@ -452,7 +526,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
             unsigned h = renum_home(id, cap);
             while (true) {
                 const int seen = atomicCAS(&tab[h].x, 0, id + 1);
-                if (seen == 0) { store_agent(&tab[h].y, atomicAdd(&s_count, 1)); return; }
+                if (seen == 0) { store_agent(&tab[h].y, ranked ? (int)local((unsigned)id) : atomicAdd(&s_count, 1)); return; }
                 if (seen == id + 1) return;
                 h = h + 1 == cap ? 0 : h + 1;
             }
@@ -474,10 +548,12 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         if (tid == 0) { enter((int)st_state); enter((int)en_state); }
         wait_stores();
         __syncthreads();
-        S = s_count;
-        SP = (int)round16(S);
-        start_loc = number_of((int)st_state);
-        end_loc = number_of((int)en_state);
+        if (!ranked) {
+            S = s_count;
+            SP = (int)round16(S);
+            start_loc = number_of((int)st_state);
+            end_loc = number_of((int)en_state);
+        }
     }
 
     if (role == 2) {
@@ -521,7 +597,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         unsigned k = ~0u;
         if (i < n_edges) {
             int e = edge_at(i);
-            unsigned p = role == 0 ? (unsigned)e_to[e] - smin : role == 1 ? (unsigned)e_from[e] - smin : slot_of((unsigned)e_emis[e]);
+            unsigned p = role == 0 ? local((unsigned)e_to[e]) : role == 1 ? local((unsigned)e_from[e]) : slot_of((unsigned)e_emis[e]);
             k = (p << KEY_POS_BITS) | (unsigned)i;
         }
         keys[i] = k;
@@ -595,7 +671,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
             unsigned p = keys[i] >> KEY_POS_BITS;
             int k = i - lower_bound_hi(keys, n_edges, p);
             int e = edge_at((int)(keys[i] & POS_MASK));
-            unsigned other = (role == 0 ? (unsigned)e_from[e] : (unsigned)e_to[e]) - smin;
+            unsigned other = local(role == 0 ? (unsigned)e_from[e] : (unsigned)e_to[e]);
             unsigned slot = slot_of((unsigned)e_emis[e]);
             ell[(size_t)k * SP + p] = make_uint2(other | (slot << 16), __float_as_uint(a.weights[e] * wscale));
         }
@@ -604,7 +680,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         uint4* crec = a.crec + edge_begin;
         for (int i = tid; i < n_edges; i += NT) {
             int e = edge_at((int)(keys[i] & POS_MASK));
-            unsigned f = (unsigned)e_from[e] - smin, t = (unsigned)e_to[e] - smin;
+            unsigned f = local((unsigned)e_from[e]), t = local((unsigned)e_to[e]);
             crec[i] = make_uint4(f | (t << 16), __float_as_uint(a.weights[e] * LOG2E), keys[i] >> KEY_POS_BITS, 0u);
         }
         int* cb = a.cbegin + goff;
@@ -631,20 +707,32 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         int dmax = 0, dmin = 0;
         for (int i = tid; i < n_edges; i += NT) {
             const int e = edge_at(i);
-            const int df = (int)((unsigned)e_to[e] - (unsigned)e_from[e]);
+            const int df = (int)local((unsigned)e_to[e]) - (int)local((unsigned)e_from[e]);
             dmax = max(dmax, df); dmin = min(dmin, df);
         }
         if (dmax > 0) atomicMax(&s_dmax, dmax);
         if (dmin < 0) atomicMin(&s_dmin, dmin);
         __syncthreads();
         dmax = s_dmax; dmin = s_dmin;
-        const int s_loc = (int)(st_state - smin), e_loc = (int)(en_state - smin);
+        const int s_loc = start_loc, e_loc = end_loc;
         // one thread per edge; the per-slot minimum / maximum is taken with LDS atomics in the
-        // memory of the sort keys, which are not needed any more once each thread has read its own
+        // memory of the sort keys (and of the distinct ids of a renumbered sequence), which is not
+        // needed any more once each thread has worked out the frames of its own edges
         constexpr int EPT = EB_MAX / NT;
-        unsigned mykey[EPT];
+        int slot_[EPT], from_[EPT], upto_[EPT];     // slot of my edges (-1: none), first and last live frame
 #pragma unroll
-        for (int j = 0; j < EPT; j++) mykey[j] = tid + j * NT < n_edges ? keys[tid + j * NT] : ~0u;
+        for (int j = 0; j < EPT; j++) {
+            slot_[j] = -1; from_[j] = 0; upto_[j] = -1;
+            if (tid + j * NT < n_edges) {
+                const unsigned key = keys[tid + j * NT];
+                const int e = edge_at((int)(key & POS_MASK));
+                const int u = (int)local((unsigned)e_from[e]), v = (int)local((unsigned)e_to[e]);
+                const int a1 = min_steps(v, e_loc, dmax, dmin);
+                slot_[j] = (int)(key >> KEY_POS_BITS);
+                from_[j] = min_steps(s_loc, u, dmax, dmin);
+                upto_[j] = a1 <= L - 1 ? L - 1 - a1 : -1;
+            }
+        }
         __syncthreads();
         int* s_tlo = (int*)keys;
         int* s_thi = (int*)keys + D_MAX;
@@ -653,13 +741,9 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < EPT; j++) {
-            if (mykey[j] != ~0u) {
-                const int e = edge_at((int)(mykey[j] & POS_MASK));
-                const int d = (int)(mykey[j] >> KEY_POS_BITS);
-                const int u = (int)((unsigned)e_from[e] - smin), v = (int)((unsigned)e_to[e] - smin);
-                const int a0 = min_steps(s_loc, u, dmax, dmin), a1 = min_steps(v, e_loc, dmax, dmin);
-                atomicMin(&s_tlo[d], a0);
-                if (a1 <= L - 1) atomicMax(&s_thi[d], L - 1 - a1);
+            if (slot_[j] >= 0) {
+                atomicMin(&s_tlo[slot_[j]], from_[j]);
+                if (upto_[j] >= 0) atomicMax(&s_thi[slot_[j]], upto_[j]);
             }
         }
         __syncthreads();
@@ -1737,7 +1821,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
     pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = g_no_band; pa.force_generic = f_too_large ? 1 : 0;
-    pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx);
+    pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx); pa.renum = (int2*)(ws + l.renum);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
     GatherArgs ga;
@@ -1746,7 +1830,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.ascending = 0;
     GenArgs gen;
     gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
-    gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx; gen.renum = (const int2*)pa.ellA;
+    gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx; gen.renum = pa.renum;
     RecArgs ra;
     ra.gen = gen;
     ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab; ra.gtab_rw = ga.gtab;
@@ -1920,7 +2004,7 @@ int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32
         FILE* f = fopen(name.c_str(), "w");
         if (!f) return I6FBW_ERR_INVALID_ARGUMENT;
         const SeqMeta& m = meta[b];
-        const bool ok = !(m.err || m.errA || m.errB);
+        const bool ok = !(m.err || m.errA || m.errB) && !(m.pad & 2);      // (no dump for renumbered state ids)
         const long long first = se[b], last = se[B + b];           // the reference walks the ids start..end
         // frame 0 is written even for an empty sequence (fbw_op.cu:177); it holds the start state only
         const int frames = !ok ? 0 : (m.L > 0 && m.n_edges > 0 ? m.L : 1);

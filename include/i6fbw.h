@@ -33,8 +33,7 @@ enum {
     I6FBW_ERR_F_TOO_LARGE = -4,           /* not returned any more */
     I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* not reported any more */
     I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* not reported any more: a sequence whose state ids span more than
-                                             2*edges+2 ids gets dense numbers for its states on the device and
-                                             takes the general path */
+                                             2*edges+2 ids gets dense numbers for its states on the device */
     I6FBW_ERR_SEQ_DEGREE = -12,           /* not reported any more */
     I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side, i6fbw_viterbi: values and back-pointers of a sequence on the
                                              general path do not fit its share of the workspace (T < 2*edges+16 with

@@ -85,14 +85,31 @@ def test_status_is_clean_for_general_path():
                                      ("monophone", dict(T=400, B=2, F=70, n_labels=(90, 100)))])
 def test_widely_spread_state_ids(oracle, how, name, kw):
     """The reference indexes its state buffers with the ids as they come, so ids need not be compact.
-    Sequences whose ids span much more than their number get dense numbers on the device (and take the
-    general path); the oracle sees the spread ids as they are."""
+    Sequences whose ids span much more than their number get dense numbers on the device (their rank
+    among the ids of the sequence) and stay on the fast kernels; the oracle sees the spread ids as they
+    are.  Ids that keep their order give the tables of the compact numbering, hence the same bits."""
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import run_cabi
     W = make_workload(name, **kw)
     edges, start_end, n_states = spread_state_ids(W.edges, W.start_end_states, W.n_states, how)
-    out, loss = check_against_oracle(oracle, (W.am_scores, edges, W.weights, start_end, W.seq_lens, n_states), bitwise=False)
-    # and it is the result of the compact numbering
-    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
-    np.testing.assert_allclose(loss, want_loss, rtol=1e-5, atol=1e-6)
+    out, loss = check_against_oracle(oracle, (W.am_scores, edges, W.weights, start_end, W.seq_lens, n_states))
+    compact_out, compact_loss = run_cabi(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states,
+                                         out_mode=cabi.OUT_NEG_LOG)
+    if how == "stride":
+        np.testing.assert_array_equal(loss, compact_loss)
+        np.testing.assert_array_equal(out, compact_out)
+    else:
+        np.testing.assert_allclose(loss, compact_loss, rtol=1e-5, atol=1e-6)
+
+
+def test_widely_spread_state_ids_of_a_large_sequence(oracle):
+    """More than 4095 edges: too many ids to sort in LDS; numbers are handed out through a table in the
+    workspace and the sequence takes the general path."""
+    W = make_workload("cart", T=5200, B=1, F=200, n_labels=(700, 700))
+    W.seq_lens[:] = W.T
+    assert W.E > 4095
+    edges, start_end, n_states = spread_state_ids(W.edges, W.start_end_states, W.n_states, "permute")
+    check_against_oracle(oracle, (W.am_scores, edges, W.weights, start_end, W.seq_lens, n_states), bitwise=False)
 
 
 def test_two_sequences_naming_the_same_states(oracle):
