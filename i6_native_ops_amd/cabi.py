@@ -20,7 +20,8 @@ STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
            "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment", "i6fbw_set_band",
            "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
-           "i6fbw_profile_enable", "i6fbw_profile_read")
+           "i6fbw_profile_enable", "i6fbw_profile_read",
+           "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode")
 
 _lib = None
 
@@ -66,6 +67,14 @@ def load():
         lib.i6fbw_build_hmm_fsa.restype = c.c_int
         lib.i6fbw_read_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.POINTER(c.c_int), c.POINTER(c.c_int)]
         lib.i6fbw_read_status.restype = c.c_int
+        lib.i6fbw_post_status.argtypes = [c.c_void_p, c.c_int, c.c_void_p]
+        lib.i6fbw_post_status.restype = c.c_int
+        lib.i6fbw_poll_status.argtypes = [c.c_int, c.POINTER(c.c_int), c.POINTER(c.c_int)]
+        lib.i6fbw_poll_status.restype = c.c_int
+        lib.i6fbw_set_status_mode.argtypes = [c.c_int]
+        lib.i6fbw_set_status_mode.restype = None
+        lib.i6fbw_get_status_mode.argtypes = []
+        lib.i6fbw_get_status_mode.restype = c.c_int
         lib.i6fbw_strerror.argtypes = [c.c_int]
         lib.i6fbw_strerror.restype = c.c_char_p
         lib.i6fbw_last_hip_error.restype = c.c_char_p
@@ -131,6 +140,22 @@ def read_status(ws_ptr, B, stream=0):
     if rc != 0:
         raise FbwError(rc)
     return int(code.value), int(seq.value)
+
+
+def post_status(ws_ptr, B, stream=0):
+    """Enqueues the status report of the last call on this workspace; nothing waits."""
+    rc = load().i6fbw_post_status(ws_ptr, B, stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def poll_status(wait=False):
+    """(code, seq) of the first problem among the reports that have arrived (all of them if ``wait``)."""
+    code, seq = ctypes.c_int(0), ctypes.c_int(-1)
+    rc = load().i6fbw_poll_status(1 if wait else 0, ctypes.byref(code), ctypes.byref(seq))
+    if rc != 0:
+        raise FbwError(rc)
+    return code.value, seq.value
 
 
 def set_overlap(mode: int) -> None:

@@ -1591,6 +1591,26 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     }
 }
 
+// Status of a call in two ints {code, sequence}: the first sequence with a reported problem, else a
+// timeout of the hand-off between kernels, else ok.  One workgroup.
+__global__ __launch_bounds__(256) void fbw_status_reduce(const SeqMeta* meta, int B, const int* sync, int* out2) {
+    __shared__ int first_bad;
+    if (threadIdx.x == 0) first_bad = 0x7fffffff;
+    __syncthreads();
+    for (int b = threadIdx.x; b < B; b += 256)
+        if (meta[b].err < 0 || meta[b].errA < 0 || meta[b].errB < 0) atomicMin(&first_bad, b);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int code = sync[0] ? I6FBW_ERR_TIMEOUT : I6FBW_OK, seq = -1;
+        if (first_bad != 0x7fffffff) {
+            const SeqMeta& m = meta[first_bad];
+            code = m.err < 0 ? m.err : (m.errA < 0 ? m.errA : m.errB);
+            seq = first_bad;
+        }
+        out2[0] = code; out2[1] = seq;
+    }
+}
+
 // Check that two streams really run at the same time (see runs_beside).
 __device__ int g_selftest[4];
 __global__ void fbw_selftest_wait() {
@@ -1745,6 +1765,37 @@ int g_no_band = 0;      // see i6fbw_set_band
 int g_overlap_mode = [] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
+}();
+
+// Status reports that travel to the host without a wait: per device a ring of pinned {code, seq}
+// slots, each with the event that follows its copy on the caller's stream.
+struct StatusRing {
+    static constexpr int SLOTS = 64;
+    int* host = nullptr;                 // SLOTS x 2 ints, pinned
+    hipEvent_t ev[SLOTS] = {};
+    bool used[SLOTS] = {};
+    int next = 0;
+    int held_code = I6FBW_OK, held_seq = -1;     // first problem seen and not yet handed to the caller
+};
+StatusRing g_status[MAX_DEVICES];
+
+// takes the result out of slot i (its event has completed or is waited for here)
+void status_collect(StatusRing& r, int i, bool wait) {
+    if (!r.used[i]) return;
+    if (wait) { if (hipEventSynchronize(r.ev[i]) != hipSuccess) return; }
+    else if (hipEventQuery(r.ev[i]) != hipSuccess) return;
+    r.used[i] = false;
+    const int code = r.host[2 * i], seq = r.host[2 * i + 1];
+    if (code != I6FBW_OK && r.held_code == I6FBW_OK) { r.held_code = code; r.held_seq = seq; }
+}
+
+// how the bindings report device-side problems: 0 not at all, 1 by waiting for every call, 2 without
+// waiting, at a later call; I6FBW_STATUS=off|sync|deferred sets the initial value (I6FBW_ASYNC=1: off)
+int g_status_mode = [] {
+    const char* e = getenv("I6FBW_STATUS");
+    if (e) return e[0] == 'o' ? 0 : (e[0] == 's' ? 1 : 2);
+    const char* a = getenv("I6FBW_ASYNC");
+    return (a && a[0] == '1') ? 0 : 2;
 }();
 
 }  // namespace
@@ -1952,6 +2003,54 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
     }
     free(host);
     return I6FBW_OK;
+}
+
+int i6fbw_post_status(void* workspace, int B, void* stream) {
+    if (!workspace || B <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    StatusRing& r = g_status[dev];
+    if (!r.host) HIP_TRY(hipHostMalloc((void**)&r.host, sizeof(int) * 2 * StatusRing::SLOTS, hipHostMallocDefault));
+    const int i = r.next;
+    r.next = (r.next + 1) % StatusRing::SLOTS;
+    status_collect(r, i, true);                  // the oldest report, if the ring has come round to it
+    if (!r.ev[i]) HIP_TRY(hipEventCreateWithFlags(&r.ev[i], hipEventDisableTiming));
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    // {code, seq} go through two unused ints of the hand-off header, which sits behind the meta records
+    int* sync = (int*)(ws + align256(sizeof(SeqMeta) * (size_t)B));
+    hipLaunchKernelGGL(fbw_status_reduce, dim3(1), dim3(256), 0, s, (const SeqMeta*)ws, B, sync, sync + 4);
+    HIP_TRY(hipGetLastError());
+    r.host[2 * i] = I6FBW_OK; r.host[2 * i + 1] = -1;
+    HIP_TRY(hipMemcpyAsync(r.host + 2 * i, sync + 4, 2 * sizeof(int), hipMemcpyDeviceToHost, s));
+    HIP_TRY(hipEventRecord(r.ev[i], s));
+    r.used[i] = true;
+    return I6FBW_OK;
+}
+
+int i6fbw_poll_status(int wait, int* code, int* seq) {
+    if (!code || !seq) return I6FBW_ERR_INVALID_ARGUMENT;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    StatusRing& r = g_status[dev];
+    for (int k = 0; k < StatusRing::SLOTS; k++) status_collect(r, (r.next + k) % StatusRing::SLOTS, wait != 0);   // oldest first
+    *code = r.held_code; *seq = r.held_seq;
+    r.held_code = I6FBW_OK; r.held_seq = -1;
+    return I6FBW_OK;
+}
+
+void i6fbw_set_status_mode(int mode) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_status_mode = mode <= 0 ? 0 : (mode == 1 ? 1 : 2);
+}
+
+int i6fbw_get_status_mode(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    return g_status_mode;
 }
 
 const char* i6fbw_strerror(int code) {

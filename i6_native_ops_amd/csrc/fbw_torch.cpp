@@ -11,6 +11,7 @@
 #include <torch/extension.h>
 
 #include "../../include/i6fbw.h"
+#include "status_report.h"
 
 namespace py = pybind11;
 
@@ -31,14 +32,6 @@ struct DebugOptions {
     CHECK_CUDA(x);           \
     CHECK_CONTIGUOUS(x);     \
     CHECK_TYPE(x, type)
-
-static bool status_check_enabled() {
-    static const bool on = [] {
-        const char* e = std::getenv("I6FBW_ASYNC");
-        return !(e && e[0] == '1');
-    }();
-    return on;
-}
 
 // fused == false: am_scores is (T, B, F), -log p, contiguous; out is (T, B, F).
 // fused == true:  am_scores is log_probs (B, T, F) with unit innermost stride; out is (B, T, F).
@@ -93,11 +86,14 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
                            (void*)stream);
     if (all_scores) i6fbw_set_band(1);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
-    if (status_check_enabled()) {
+    // a dump reads the workspace on the host anyway: such a call waits for its own status
+    if (dump && i6fbw_get_status_mode() == 2) {
         int code = 0, seq = -1;
         rc = i6fbw_read_status(workspace.data_ptr(), B, (void*)stream, &code, &seq);
         TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
         TORCH_CHECK(code == I6FBW_OK, "NativeOp: fbw: sequence ", seq, ": ", i6fbw_strerror(code));
+    } else {
+        i6_status::report("fbw", workspace.data_ptr(), B, (void*)stream);
     }
     if (dump && dump->dump_alignment) {
         // as fbw_op.cu:361-364
@@ -153,6 +149,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("debug_options") = DebugOptions());
     m.def("fbw_fused", &fbw_fused,
           "fbw_loss in one call: log_probs (B, T, F) -> [gradient w.r.t. log_probs = -posterior (B, T, F), loss (T, B)]");
+    i6_status::bind(m);
     m.def("fbw_posterior", &fbw_posterior,
           "Same as fbw but the first result holds the posteriors themselves (exp(-out)) with 0 in the holes");
 }

@@ -10,6 +10,7 @@
 #include <torch/extension.h>
 
 #include "../../include/i6fbw.h"
+#include "status_report.h"
 
 // Same checks and messages as CHECK_INPUT (common/returnn_definitions.h:93-99).
 #define CHECK_CUDA(x) TORCH_CHECK(x.device().is_cuda(), #x " must be a CUDA tensor")
@@ -67,13 +68,7 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
                        T, B, F, E, (int)num_states, alignment.data_ptr<int32_t>(), alignment.stride(dt),
                        alignment.stride(db), scores.data_ptr<float>(), workspace.data_ptr(), ws_bytes, (void*)stream);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fast_viterbi: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
-    const char* async = std::getenv("I6FBW_ASYNC");
-    if (!(async && async[0] == '1')) {
-        int code = 0, seq = -1;
-        rc = i6fbw_read_status(workspace.data_ptr(), B, (void*)stream, &code, &seq);
-        TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fast_viterbi: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
-        TORCH_CHECK(code == I6FBW_OK, "NativeOp: fast_viterbi: sequence ", seq, ": ", i6fbw_strerror(code));
-    }
+    i6_status::report("fast_viterbi", workspace.data_ptr(), B, (void*)stream);
     return {alignment, scores};
 }
 
@@ -92,6 +87,7 @@ std::vector<torch::Tensor> fast_viterbi_batch_major(torch::Tensor& log_probs, to
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fast_viterbi", &fast_viterbi, "Fast Viterbi routine (MI355X)");
+    i6_status::bind(m);
     m.def("fast_viterbi_batch_major", &fast_viterbi_batch_major,
           "align_viterbi in one call: log_probs (B, T, F) -> [alignment (B, T) int32, scores (B,)]");
 }

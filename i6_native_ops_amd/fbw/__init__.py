@@ -5,6 +5,10 @@ Same public surface as ``i6_native_ops.fbw`` (i6_native_ops/fbw/__init__.py:27-6
 ``fbw`` and ``DebugOptions``.  The extension is built ahead of time by
 ``i6_native_ops_amd/build.py``; nothing is compiled at import, and there is no CPU or eager
 fallback: without the built HIP library the import fails.
+
+Problems only the device can see (an index out of range) do not make a call wait for the device:
+they are raised by a later call or by ``check_status()``; ``set_status_mode("sync")`` makes every
+call wait and raise for itself (the reference has undefined behaviour there).
 """
 from typing import Tuple
 
@@ -88,4 +92,7 @@ def fbw_loss_unfused(log_probs, fsa, seq_lens):
     return FastBaumWelchLoss.apply(neg_log_probs, fsa, seq_lens)
 
 
-__all__ = ["fbw_loss", "fbw_loss_unfused", "FastBaumWelchLoss", "core"]
+set_status_mode = core.set_status_mode
+check_status = core.check_status
+
+__all__ = ["fbw_loss", "fbw_loss_unfused", "FastBaumWelchLoss", "core", "set_status_mode", "check_status"]

@@ -7,7 +7,7 @@
  * entry points below are what a binding for that function needs: plain
  * pointers and sizes, no torch types.  All data pointers are DEVICE pointers
  * owned by the caller; the library never allocates or frees device memory and
- * never synchronises the device (i6fbw_read_status excepted).
+ * never synchronises the device (i6fbw_read_status and i6fbw_poll_status(1, ...) excepted).
  */
 #ifndef I6FBW_H
 #define I6FBW_H
@@ -124,6 +124,30 @@ int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_st
  * paths (fbw_op.cu:287-290, returnn_definitions.h:114-123) with a status.
  */
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq);
+
+/*
+ * The same report without a wait, for callers that must not stall the host (a training loop that
+ * keeps the device queue full): i6fbw_post_status enqueues, on `stream`, a one-workgroup reduction of
+ * the status of the last call that used this workspace with batch size B and its copy into pinned
+ * host memory owned by the library (64 reports per device can be in flight; the call waits for the
+ * oldest one if all are).  i6fbw_poll_status hands back the first problem among the reports of the
+ * current device that have arrived (wait == 0) or among all of them after waiting for them
+ * (wait != 0), and forgets it; *code is I6FBW_OK if there is none.  The workspace may be reused or
+ * released in stream order after i6fbw_post_status returns.  No counterpart in the reference, whose
+ * device-side problems are undefined behaviour (fbw_op.cu:287-290).
+ */
+int i6fbw_post_status(void* workspace, int B, void* stream);
+int i6fbw_poll_status(int wait, int* code, int* seq);
+
+/*
+ * How the PyTorch bindings built on this library report device-side problems: 0 not at all, 1 by
+ * waiting for every call (i6fbw_read_status; the error belongs to the call that raises it), 2 without
+ * waiting (i6fbw_post_status / i6fbw_poll_status; the error is raised by a later call or by the
+ * bindings' check_status()).  Initial value: 2, or what the environment variable I6FBW_STATUS
+ * (off | sync | deferred) says.
+ */
+void i6fbw_set_status_mode(int mode);
+int i6fbw_get_status_mode(void);
 
 /*
  * Best path (Viterbi alignment) on the same automaton description.  Replaces fast_viterbi_cuda

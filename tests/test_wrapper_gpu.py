@@ -100,6 +100,7 @@ def test_device_side_status_is_reported():
     """Indices the reference would read out of bounds with, and automata beyond the supported
     size, surface as RuntimeError instead of the reference's abort()/undefined behaviour."""
     from i6_native_ops_amd.fbw import core
+    core.set_status_mode("sync")        # every call waits for its own result (the fixture of conftest.py restores the default)
     log_probs, (n, edges, weights, se), seq_lens = _fixture_tensors()
     am = log_probs.detach().neg().transpose(0, 1).contiguous()
     bad = edges.clone()
@@ -238,3 +239,38 @@ def test_two_host_threads_on_their_own_streams(overlap):
         assert not failures, failures
     finally:
         cabi.set_overlap(-1)
+
+
+def test_deferred_status_does_not_wait_and_is_raised_later():
+    """Default mode: a call with an index out of range returns at once, its sequence holds NaN, and the
+    problem is raised by check_status() or by the next call that finds the report arrived; after that
+    the library is clean again.  Mode 'off' raises nothing."""
+    from i6_native_ops_amd.fbw import core
+    from i6_native_ops_amd.fast_viterbi import core as vcore
+    assert core.get_status_mode() == "deferred" and vcore.get_status_mode() == "deferred"
+    log_probs, (n, edges, weights, se), seq_lens = _fixture_tensors()
+    am = log_probs.detach().neg().transpose(0, 1).contiguous()
+    bad = edges.clone()
+    bad[2, 1] = 5                       # emission index >= F
+    out, loss = core.fbw(am, bad, weights, se, seq_lens, n)        # no exception here
+    assert torch.isnan(loss).all()
+    with pytest.raises(RuntimeError, match="an earlier call reported: sequence 0: .*index out of range"):
+        core.check_status()
+    core.check_status()                 # reported once
+    # raised by a later call, of either module, once the report has arrived
+    core.fbw(am, bad, weights, se, seq_lens, n)
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="an earlier call reported"):
+        vcore.fast_viterbi(am, edges, weights, se, seq_lens, n)
+    out, loss = core.fbw(am, edges, weights, se, seq_lens, n)
+    core.check_status()
+    assert torch.isfinite(loss).all()
+    # many calls in flight: more than the ring of reports holds
+    for _ in range(150):
+        core.fbw(am, edges, weights, se, seq_lens, n)
+    core.check_status()
+    core.set_status_mode("off")
+    core.fbw(am, bad, weights, se, seq_lens, n)
+    torch.cuda.synchronize()
+    core.fbw(am, edges, weights, se, seq_lens, n)
+    core.check_status()
