@@ -1779,14 +1779,16 @@ struct StatusRing {
 };
 StatusRing g_status[MAX_DEVICES];
 
-// takes the result out of slot i (its event has completed or is waited for here)
-void status_collect(StatusRing& r, int i, bool wait) {
-    if (!r.used[i]) return;
-    if (wait) { if (hipEventSynchronize(r.ev[i]) != hipSuccess) return; }
-    else if (hipEventQuery(r.ev[i]) != hipSuccess) return;
+// takes the result out of slot i (its event has completed or is waited for here); false if the
+// report is still on its way
+bool status_collect(StatusRing& r, int i, bool wait) {
+    if (!r.used[i]) return true;
+    if (wait) { if (hipEventSynchronize(r.ev[i]) != hipSuccess) return false; }
+    else if (hipEventQuery(r.ev[i]) != hipSuccess) return false;
     r.used[i] = false;
     const int code = r.host[2 * i], seq = r.host[2 * i + 1];
     if (code != I6FBW_OK && r.held_code == I6FBW_OK) { r.held_code = code; r.held_seq = seq; }
+    return true;
 }
 
 // how the bindings report device-side problems: 0 not at all, 1 by waiting for every call, 2 without
@@ -2037,7 +2039,10 @@ int i6fbw_poll_status(int wait, int* code, int* seq) {
     if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
     std::lock_guard<std::mutex> lock(g_mutex);
     StatusRing& r = g_status[dev];
-    for (int k = 0; k < StatusRing::SLOTS; k++) status_collect(r, (r.next + k) % StatusRing::SLOTS, wait != 0);   // oldest first
+    // oldest first; reports arrive in the order of the calls (on one stream), so the first one that
+    // is still on its way ends the search: a poll costs one or two event queries, not sixty-four
+    for (int k = 0; k < StatusRing::SLOTS; k++)
+        if (!status_collect(r, (r.next + k) % StatusRing::SLOTS, wait != 0)) break;
     *code = r.held_code; *seq = r.held_seq;
     r.held_code = I6FBW_OK; r.held_seq = -1;
     return I6FBW_OK;
