@@ -1984,8 +1984,16 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     return I6FBW_OK;
 }
 
+// a stream that is being captured into a graph can neither be waited for nor carry the events of
+// the status ring: no report from there
+static bool is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+}
+
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq) {
     if (!workspace || B <= 0 || !code || !seq) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (is_capturing((hipStream_t)stream)) { *code = I6FBW_OK; *seq = -1; return I6FBW_OK; }
     // the meta records sit at the start of the workspace, the abort flag of the hand-off area right
     // behind them: one copy brings both
     const size_t flag_at = align256(sizeof(SeqMeta) * (size_t)B);
@@ -2009,6 +2017,7 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
 
 int i6fbw_post_status(void* workspace, int B, void* stream) {
     if (!workspace || B <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (is_capturing((hipStream_t)stream)) return I6FBW_OK;
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;

@@ -8,6 +8,7 @@
 #pragma once
 #include <string>
 
+#include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
 #include "../../include/i6fbw.h"
@@ -17,6 +18,9 @@ namespace i6_status {
 inline void report(const char* op, void* workspace, int B, void* stream) {
     const int mode = i6fbw_get_status_mode();
     if (mode == 0) return;
+    // while the stream is being captured into a graph nothing may be waited for or queried
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return;
     int code = 0, seq = -1;
     if (mode == 1) {
         const int rc = i6fbw_read_status(workspace, B, stream, &code, &seq);

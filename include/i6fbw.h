@@ -122,6 +122,8 @@ int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_st
  * used this workspace with batch size B: *code is I6FBW_OK or one of the device-side codes, *seq
  * the first sequence it was seen on.  Replaces the reference's abort()/assert
  * paths (fbw_op.cu:287-290, returnn_definitions.h:114-123) with a status.
+ * On a stream that is being captured into a graph nothing can be waited for: the call then
+ * reports I6FBW_OK without looking (and i6fbw_post_status enqueues nothing).
  */
 int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int* seq);
 

@@ -274,3 +274,42 @@ def test_deferred_status_does_not_wait_and_is_raised_later():
     torch.cuda.synchronize()
     core.fbw(am, edges, weights, se, seq_lens, n)
     core.check_status()
+
+
+@pytest.mark.parametrize("mode", ["deferred", "sync"])
+def test_graph_capture_through_the_binding(mode):
+    """fbw_loss forward and backward inside torch.cuda.graph: the binding reports no status from a
+    capturing stream (nothing there can be waited for or queried), and replays give the eager result."""
+    from i6_native_ops_amd.fbw import core, fbw_loss
+    core.set_status_mode(mode)
+    W = make_workload("cart", T=60, B=4, F=200)
+    dev = torch.device("cuda:0")
+    fsa = (W.n_states, torch.from_numpy(W.edges).to(dev), torch.from_numpy(W.weights).to(dev),
+           torch.from_numpy(W.start_end_states).to(dev))
+    seq_lens = torch.from_numpy(W.seq_lens).to(dev)
+    static_in = torch.from_numpy(-W.am_scores).transpose(0, 1).contiguous().to(dev).requires_grad_(True)
+    eager = fbw_loss(static_in, fsa, seq_lens)
+    eager.sum().backward()
+    want_loss, want_grad = eager.detach().clone(), static_in.grad.detach().clone()
+    del eager                                                # its autograd graph belongs to the default stream
+    static_in.grad = None
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                                   # warm-up on the side stream
+            fbw_loss(static_in, fsa, seq_lens).sum().backward()
+            static_in.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loss = fbw_loss(static_in, fsa, seq_lens)
+        loss.sum().backward()
+    for _ in range(3):
+        loss.fill_(-1.0)
+        static_in.grad.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(loss.detach(), want_loss)
+        assert torch.equal(static_in.grad, want_grad)
+    core.check_status()
