@@ -241,7 +241,7 @@ struct PrepArgs {
     int T, B, F, E, n_states;
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
-    int force_generic;  // F is too large for the emission bitmap or the row image: every sequence takes the general path
+    int force_generic;  // F is too large for the emission bitmap: every sequence takes the general path
     int2* renum;        // renumbering tables, two entries per state of room (see local_state)
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
 };
@@ -1284,6 +1284,7 @@ struct CombArgs {
     float* out; float* sum_output;
     long long ost_t, ost_b;      // element strides of out over frames and sequences
     int* sync;
+    int tile_w;                  // 0: the row image holds the whole row; else its width in floats (a multiple of 32), see finish_row
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1339,6 +1340,21 @@ __device__ inline void stream_image_row(float* row, int F, const float4a* lds4, 
     if (threadIdx.x < 8) {
         const int i = threadIdx.x < 4 ? 4 * (ch_lo - 1) + threadIdx.x : 4 * ch_hi + threadIdx.x - 4;
         if (i >= a && i < a + F && (i < 4 * ch_lo || i >= 4 * ch_hi)) base[i] = image[i];
+    }
+}
+
+// chunks [c0, c1) of the line-aligned view of a row (base + 4 * chunk); chunk ch sits at lds4[ch - cofs]
+__device__ inline void stream_tile(float* base, const int c0, const int c1, const int cofs, const float4a* lds4) {
+    constexpr int U = 4;
+    for (int ch0 = c0 + threadIdx.x; ch0 < c1; ch0 += U * COMB_THREADS) {
+        float4a v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = lds4[min(ch0 + u * COMB_THREADS, c1 - 1) - cofs];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int ch = ch0 + u * COMB_THREADS;
+            if (ch < c1) I6_ROW_STORE(v[u], (float4a*)(base + 4 * ch));
+        }
     }
 }
 
@@ -1446,7 +1462,9 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
     const float psign = a.out_mode == I6FBW_OUT_NEG_PROB ? -1.f : 1.f;
 
     float* image = (float*)lds4;
-    const int F4 = (F + 32 + 3) >> 2;     // the image is shifted by the row's offset within its 128-byte line
+    // the image is shifted by the row's offset within its 128-byte line; rows too long for LDS go
+    // through it in tiles of tile_w floats
+    const int F4 = a.tile_w ? a.tile_w >> 2 : (F + 32 + 3) >> 2;
     float* xs = image + 4 * F4;
     for (int i = tid; i < F4; i += COMB_THREADS) lds4[i] = (float4a){hole, hole, hole, hole};
     int a_prev = -1;                      // image shift of the previous frame
@@ -1471,6 +1489,39 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
         const float inv = dead ? 0.f : psign / tot;
         float* orow = a.out + t * a.ost_t + b * a.ost_b;
         const int sh = row_misalign(orow);
+        if (a.tile_w) {
+            // Row longer than the image: tile after tile of the line-aligned view of the row (positions
+            // sh .. sh+F-1 of base = orow - sh).  The slots are ordered by emission index, but every
+            // thread simply looks which of its slots fall into the tile; after the tile has gone out
+            // their positions get the hole value back.
+            auto value = [&](int js) -> float {
+                if (prob) return sd[js] * inv;
+                return (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+            };
+            float* base = orow - sh;
+            const int W = a.tile_w, P = sh + F;
+            const int ch_lo = (sh + 3) >> 2, ch_hi = P >> 2;             // chunks that lie completely inside the row
+            for (int p0 = 0; p0 < P; p0 += W) {
+                const int p1 = min(p0 + W, P);
+                for (int js = 0; js < nslot_regs; js++) {
+                    const int p = sh + em[js];
+                    if (tid + js * COMB_THREADS < D && p >= p0 && p < p1) image[p - p0] = value(js);
+                }
+                __syncthreads();
+                stream_tile(base, max(p0 >> 2, ch_lo), min((p0 + W) >> 2, ch_hi), p0 >> 2, lds4);
+                if (tid < 8) {                                            // the floats of the two cut chunks of the row
+                    const int i = tid < 4 ? 4 * (ch_lo - 1) + tid : 4 * ch_hi + tid - 4;
+                    if (i >= sh && i < P && (i < 4 * ch_lo || i >= 4 * ch_hi) && i >= p0 && i < p1) base[i] = image[i - p0];
+                }
+                __syncthreads();
+                for (int js = 0; js < nslot_regs; js++) {
+                    const int p = sh + em[js];
+                    if (tid + js * COMB_THREADS < D && p >= p0 && p < p1) image[p - p0] = hole;
+                }
+                __syncthreads();
+            }
+            return;
+        }
         if (a_prev >= 0 && a_prev != sh) {
             for (int js = 0; js < nslot_regs; js++)
                 if (tid + js * COMB_THREADS < D) image[a_prev + em[js]] = hole;
@@ -1759,6 +1810,7 @@ struct StageTimer {
 };
 
 size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
+constexpr int COMB_TILE_W = 12288;     // floats of a row that go through LDS at a time when the row does not fit: three workgroups per unit
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
 int g_no_band = 0;      // see i6fbw_set_band
@@ -1833,10 +1885,13 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
     const Layout l = make_layout(T, B, E);
     if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
-    // too many emission classes for the LDS bitmap of the preparation or the LDS row image of the
-    // dense write: every sequence takes the general path
-    const bool f_too_large = F > F_BITMAP_MAX || comb_lds_bytes(F) > 160 * 1024 - 256;
-    const size_t comb_lds = f_too_large ? 64 : comb_lds_bytes(F);
+    // too many emission classes for the LDS bitmap of the preparation: every sequence takes the general path
+    const bool f_too_large = F > F_BITMAP_MAX;
+    // rows too long for the LDS image of the dense write go through it in tiles; so do rows of more
+    // than two tiles that would still fit (the smaller image leaves room for three workgroups on a
+    // compute unit instead of one or two: 1-2 % faster)
+    const bool tiled = comb_lds_bytes(F) > 160 * 1024 - 256 || F > 2 * COMB_TILE_W;
+    const size_t comb_lds = tiled ? (size_t)COMB_TILE_W * 4 + (size_t)COMB_XS * 4 : comb_lds_bytes(F);
 
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
@@ -1895,6 +1950,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     ca.meta = meta; ca.crec = pa.crec; ca.cbegin = pa.cbegin; ca.demis = pa.demis;
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
+    ca.tile_w = tiled ? COMB_TILE_W : 0;
     // More recursion workgroups than compute units: the instance of which two fit on a unit -- unless
     // the sequences can be longer than 4096 frames, which only the other instance runs in double
     // precision (recurse_workgroup); it then takes two rounds.

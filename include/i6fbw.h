@@ -26,8 +26,8 @@ enum {
     I6FBW_ERR_WORKSPACE_TOO_SMALL = -2,
     I6FBW_ERR_LAUNCH = -3,             /* a HIP launch failed; see i6fbw_last_hip_error() */
     /* Sequences beyond the capacity of the fast kernels (more than 8192 edges, 4096 states or 4096
-       distinct emissions in one sequence, more than 15 edges into or out of a state, F beyond about
-       36 000 for i6fbw_run / 131 072 for i6fbw_viterbi) are not refused: they take a general path
+       distinct emissions in one sequence, more than 15 edges into or out of a state, F beyond
+       131 072) are not refused: they take a general path
        that has no such limits and runs at a fraction of the speed.  The size codes remain for the
        one case that path cannot hold either. */
     I6FBW_ERR_F_TOO_LARGE = -4,           /* not returned any more */

@@ -62,12 +62,42 @@ def test_large_sequences(oracle, kind):
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=4, bitwise=False)
 
 
-@pytest.mark.parametrize("F", [40000, 140000])
+@pytest.mark.parametrize("F", [24576, 24577, 49153, 100003, 131072, 140000])
 def test_many_emission_classes(oracle, F):
-    """F beyond the LDS row image (about 36 000) and beyond the emission bitmap (131 072): all sequences
-    take the general path."""
+    """Long rows (F beyond 24 576) go through the LDS row image of the dense write in tiles of 12 288 floats,
+    still on the fast kernels with their fixed summation order; beyond the emission bitmap of the
+    preparation (131 072) all sequences take the general path."""
     W = make_workload("cart", T=60, B=3, F=F, n_labels=(10, 15))
-    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), bitwise=False)
+    # emission classes at both ends of the rows and on tile boundaries
+    for k, em in enumerate([0, 1, F - 1, F - 2, 12287, 12288, 12289, 24575, 24576]):
+        if em < F:
+            W.edges[2, 3 * k] = em
+    check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), bitwise=F <= 131072)
+
+
+@pytest.mark.parametrize("out_mode", ["neg_log", "neg_prob"])
+def test_tiled_rows_in_the_fused_layout(oracle, out_mode):
+    """Long rows in (B, T, F) order, every row at another offset within its 128-byte line (F odd)."""
+    import torch
+    from i6_native_ops_amd.fbw import fbw_loss, core
+    W = make_workload("ctc", T=30, B=5, F=45001)
+    dev = torch.device("cuda:0")
+    fsa = (W.n_states, torch.from_numpy(W.edges).to(dev), torch.from_numpy(W.weights).to(dev),
+           torch.from_numpy(W.start_end_states).to(dev))
+    seq_lens = torch.from_numpy(W.seq_lens).to(dev)
+    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    if out_mode == "neg_prob":
+        log_probs = torch.from_numpy(-W.am_scores).transpose(0, 1).contiguous().to(dev).requires_grad_(True)
+        loss = fbw_loss(log_probs, fsa, seq_lens)
+        loss.sum().backward()
+        np.testing.assert_allclose(loss.detach().cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(-log_probs.grad.transpose(0, 1).cpu().numpy(), np.exp(-want_out.astype(np.float64)), rtol=0, atol=1e-4)
+    else:
+        out, loss = core.fbw(torch.from_numpy(W.am_scores).to(dev), fsa[1], fsa[2], fsa[3], seq_lens, W.n_states)
+        np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
+        out = out.cpu().numpy()
+        assert (np.isposinf(out) == np.isposinf(want_out)).all()
+        np.testing.assert_allclose(np.exp(-out.astype(np.float64)), np.exp(-want_out.astype(np.float64)), rtol=0, atol=1e-4)
 
 
 def test_status_is_clean_for_general_path():
