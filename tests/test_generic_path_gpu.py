@@ -1,6 +1,6 @@
 """Automata beyond the capacity of the fast kernels (more than 15 edges into or out of a state,
 more than 8192 edges, 4096 states or 4096 distinct emissions in one sequence, more emission
-classes than the LDS row image holds) take the general path inside the same kernels.  Same parity
+classes than the preparation's bitmap holds) take the general path inside the same kernels.  Same parity
 bar as everything else, under both schedules, also mixed with ordinary sequences in one batch."""
 import numpy as np
 import pytest
