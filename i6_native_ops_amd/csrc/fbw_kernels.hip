@@ -32,6 +32,7 @@
 #include <cmath>
 #include <cstdio>
 #include <mutex>
+#include <type_traits>
 #include <string>
 #include <vector>
 
@@ -878,7 +879,8 @@ template <typename ST> __device__ __forceinline__ ST state_min(ST a, ST b) { ret
 // constrained that the states carrying the posterior mass sit far from the frame minimum (their
 // values would lose precision in float, frame after frame).  exp2 / log2 always work in float on
 // differences, which are small; rows go to the workspace as float either way.
-template <bool SYNC, int THREADS, int J, int KT, typename ST>
+// NJ: how many of the J rounds (states tid + j*THREADS) hold a state for this wave
+template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ>
 __device__ __forceinline__ void recurse_step(const int i, const int SP, const char* stc, ST* stn,
                                              const char* amc, float* wmin,
                                              const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
@@ -895,7 +897,7 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
     }
     float rmin = INF_F;
 #pragma unroll
-    for (int j = 0; j < J; j++) {
+    for (int j = 0; j < NJ; j++) {
         const int s = tid + j * THREADS;
         ST v[KT];
         ST mn = (ST)INF_F;
@@ -921,6 +923,18 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
     }
     step_end<SYNC>(i, cur);
+}
+
+// all steps of a wave that has states in NJ of its J rounds
+template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ>
+__device__ __forceinline__ void recurse_time_loop(const int SP, ST* st0, ST* st1, const float* am0, const float* am1, float* wmin,
+                                                  const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
+                                                  const float (&ew)[J][KT], RecCursor& cur) {
+    for (int i = 0; i < cur.nsteps; i += 2) {
+        recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
+        if (i + 1 < cur.nsteps)
+            recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
+    }
 }
 
 // common prologue of the compute waves: initial state vector, row 0 of the workspace, cursor
@@ -989,15 +1003,22 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
     if (tid < THREADS / 64) wmin[tid] = INF_F;
     RecCursor cur;
     recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
-    // Waves without a state leave: they would only compete with the others for issue slots on
-    // their SIMD, and a barrier counts the waves that are still there.  Their entries of wmin keep
-    // the +inf written above.
-    if (J == 1 && (tid & ~63) >= SP) return;
-    for (int i = 0; i < cur.nsteps; i += 2) {
-        recurse_step<SYNC, THREADS, J, KT, ST>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
-        if (i + 1 < cur.nsteps)
-            recurse_step<SYNC, THREADS, J, KT, ST>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
-    }
+    // Rounds of this wave that hold a state at all (the cells of the others keep the +inf of the
+    // start-up); the time loop is instantiated for that number, so that the LDS reads of all its
+    // rounds are issued together.  Waves without a state leave: they would only compete with the
+    // others for issue slots on their SIMD, and a barrier counts the waves that are still there.
+    // Their entries of wmin keep the +inf written above.
+    const int first = tid & ~63;
+    const int nj = first >= SP ? 0 : min(J, (SP - first + THREADS - 1) / THREADS);
+    if (nj == 0) return;
+    // (only in the instance for small batches: the one of which two workgroups share a compute unit
+    // has no registers to spare for more loop bodies)
+    constexpr bool PER_ROUND = THREADS == REC_THREADS;
+    if (!PER_ROUND) recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
+    else if (J == 1 || nj == 1) recurse_time_loop<SYNC, THREADS, J, KT, ST, 1>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
+    else if (nj == 2) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 2 ? 2 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
+    else if (nj == 3) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 3 ? 3 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
+    else recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
 }
 
 // Fallback for the largest sequences: same arithmetic, edge tables re-read from memory each frame
@@ -1719,6 +1740,7 @@ struct Pipeline {
     hipStream_t sP = nullptr, sR = nullptr;
     hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneR = nullptr;
     int n_cu = 256;
+    int dense_regs = 0;       // vector registers per lane of fbw_recurse_dense<true>, as built
     // caller streams that were checked against the recursion stream: do kernels on the two run at
     // the same time?
     std::vector<std::pair<hipStream_t, bool>> checked;
@@ -1753,6 +1775,9 @@ int pipeline_init(Pipeline& p) {
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    hipFuncAttributes attr;
+    HIP_TRY(hipFuncGetAttributes(&attr, (const void*)fbw_recurse_dense<true>));
+    p.dense_regs = attr.numRegs;
     p.ready = true;
     return I6FBW_OK;
 }
@@ -1913,6 +1938,10 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
     if (2 * B > (T <= 4096 ? 2 : 1) * P.n_cu) overlap = false;
+    // Two workgroups of the dense instance are four waves per SIMD: beyond 104 registers each they
+    // leave no room for the gather's waves, which they wait for.  (The compiler is asked for 96; how
+    // close it gets depends on its version.)
+    if (2 * B > P.n_cu && P.dense_regs > 104) overlap = false;
     if (overlap) {
         // under stream capture: one stream, no in-memory waits between kernels, no synchronisation
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
