@@ -1,20 +1,40 @@
 """Shared helpers of the test-suite: the reference's own fixture, a brute-force
 path enumerator and small random automata."""
 import itertools
+import json
+import os
 
 import numpy as np
 
 
+def golden(name):
+    """One of the reference's own test vectors, kept as data in tests/golden/reference_fixtures.json."""
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_fixtures.json")) as f:
+        return json.load(f)[name]
+
+
+def _golden_arrays(name, sign):
+    g = golden(name)
+    p = np.array(g["probabilities"], dtype=np.float32)
+    am = (sign * np.log(p))[:, None, :].astype(np.float32)      # [T,B,F]
+    edges = np.array(g["edges"], dtype=np.int32).T.copy()
+    weights = np.array(g["weights"], dtype=np.float32)
+    start_end = np.array(g["start_end_states"], dtype=np.int32)
+    return am, edges, weights, start_end, np.array(g["seq_lens"], dtype=np.int32), int(g["num_states"])
+
+
 def reference_fixture(seq_len=5):
     """The one FBW fixture the reference holds (test/fbw.py:9-41): B=1, T=5, F=2,
-    two states, three edges, all weights 1."""
-    p = np.array([[0.9, 0.1], [0.9, 0.1], [0.4, 0.6], [0.1, 0.9], [0.1, 0.9]], dtype=np.float32)
-    am = (-np.log(p))[:, None, :].astype(np.float32)            # [T,B,F]
-    edges = np.array([[0, 0, 0, 0], [0, 1, 0, 0], [1, 1, 1, 0]], dtype=np.int32).T.copy()
-    weights = np.ones(3, dtype=np.float32)
-    start_end = np.array([[0], [1]], dtype=np.int32)
-    seq_lens = np.array([seq_len], dtype=np.int32)
-    return am, edges, weights, start_end, seq_lens, 2
+    two states, three edges, all weights 1; scores are -log p."""
+    am, edges, weights, start_end, seq_lens, n = _golden_arrays("fbw", -1.0)
+    seq_lens[:] = seq_len
+    return am, edges, weights, start_end, seq_lens, n
+
+
+def reference_viterbi_fixture():
+    """test/fast_viterbi.py:9-35: the same automaton with scores log p, and the alignment the
+    reference's test expects."""
+    return _golden_arrays("fast_viterbi", 1.0), np.array(golden("fast_viterbi")["expected"]["alignment"], dtype=np.int32)
 
 
 def brute_force(am, edges, weights, start_end, seq_lens, n_states):

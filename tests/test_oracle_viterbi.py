@@ -4,17 +4,14 @@ and the low-temperature limit of the full-sum oracle."""
 import numpy as np
 import pytest
 
+from tests.helpers import golden
 from tests.helpers import random_fsa
 
 
 def viterbi_fixture():
     """test/fast_viterbi.py:9-35: B=1, T=5, F=2, two states, three edges, all weights 1."""
-    p = np.array([[0.9, 0.1], [0.9, 0.1], [0.4, 0.6], [0.1, 0.9], [0.1, 0.9]], dtype=np.float32)
-    am = np.log(p)[:, None, :].astype(np.float32)
-    edges = np.array([[0, 0, 0, 0], [0, 1, 0, 0], [1, 1, 1, 0]], dtype=np.int32).T.copy()
-    weights = np.ones(3, dtype=np.float32)
-    start_end = np.array([[0], [1]], dtype=np.int32)
-    return am, edges, weights, start_end, np.array([5], dtype=np.int32), 2
+    from tests.helpers import reference_viterbi_fixture
+    return reference_viterbi_fixture()[0]
 
 
 def all_paths(am, edges, weights, start_end, seq_lens, b):
@@ -41,7 +38,7 @@ def all_paths(am, edges, weights, start_end, seq_lens, b):
 def test_reference_vector(oracle):
     """test/fast_viterbi.py:37-42 expects [0, 0, 1, 1, 1]; the score follows from the five factors."""
     align, scores = oracle.viterbi_oracle(*viterbi_fixture())
-    assert align[:, 0].tolist() == [0, 0, 1, 1, 1]
+    assert align[:, 0].tolist() == golden("fast_viterbi")["expected"]["alignment"]
     assert scores[0] == pytest.approx(5.0 + np.log(0.9 * 0.9 * 0.6 * 0.9 * 0.9), rel=1e-6)
 
 
