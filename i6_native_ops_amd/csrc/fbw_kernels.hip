@@ -59,6 +59,8 @@ constexpr int RENORM = 8;             // frames between renormalisations of the 
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
 constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of the combine kernel
+constexpr int COMB_MID_EDGES = 4096;  // up to here a combine workgroup keeps the edges of its sequence in registers ...
+constexpr int COMB_MID_SLOTS = 2048;  // ... and the distinct emissions of the sequence spread over its threads' registers
 constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup
 constexpr int REC_LOADERS = 1;        // loader waves beside them
 constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
@@ -1188,7 +1190,9 @@ constexpr int REC_LDS_FLOATS_F32 = 2 * D_MAX + 2 * (S_MAX + 16) + 32 + 8;
 constexpr int REC_LDS_FLOATS_F64 = 2 * D_MAX + 4 * (S_MAX + 16) + 32 + 8;
 
 // the compute threads' part for one state type; the loader waves do not depend on it
-template <bool SYNC, int T_, typename ST>
+// ONE: whether sequences with one state per thread can arrive here with this state type (they are
+// not instantiated otherwise: fewer loop bodies in a kernel give the remaining ones better code)
+template <bool SYNC, int T_, typename ST, bool ONE>
 __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int cls,
                                                  ST* st0, ST* st1, const float* am0, const float* am1, float* wmin) {
     const int K = dir ? m.Kout : m.Kin;
@@ -1198,7 +1202,7 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
     constexpr bool F32 = sizeof(ST) == 4;
     if (K > KMAX) {
         recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
-    } else if (cls == 1) {
+    } else if (ONE && cls == 1) {
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
@@ -1226,6 +1230,11 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
     // gather or combine waves
     __builtin_amdgcn_s_setprio(3);
+    // In the schedule in which gather and dense write run at the same time the workgroup also claims
+    // the registers that would let their waves move in beside its own: the nine waves then hold 504
+    // (one SIMD) or 336 of a SIMD's 512 registers, as much as three waves per SIMD allow.  Measured on
+    // the headline workload: with the 142 registers the code needs, 0.575 ms per call; with 168, 0.553.
+    if (SYNC && !DENSE) asm volatile("v_mov_b32 v167, 0" ::: "v167");
     if (SYNC) {
         // This kernel is started beside the preparation, so that its large workgroups are placed
         // while the machine is still empty: report the placement (see fbw_gate), wait until all
@@ -1264,17 +1273,21 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
         else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
         return;
     }
-    // Double-precision state vectors where float would show in the posteriors: sequences with fewer
-    // than five frames for every three states (the alignment is so constrained that the states
-    // which matter sit far from the frame minimum; 1100 states in 1055 frames reach 1.4e-4 in
-    // float) and sequences of more than 4096 frames (rounding accumulates from frame to frame;
-    // 20 000 frames reach 3e-4 in float).  The dense instance has no room for them in LDS.
-    const bool wide = !DENSE && (5LL * m.S > 3LL * m.L || m.L > 4096);
+    // Double-precision state vectors where float would show in the posteriors.  State values are
+    // relative to the frame minimum, and the states that carry the posterior mass can sit a
+    // hundred units and more above it; float then loses a little in every frame (a CTC automaton of
+    // 116 labels over 764 frames reached 1.05e-4 on the posteriors, 1.2e-5 in double; 1100 states in
+    // 1055 frames 1.4e-4; 20 000 frames through 100 states 3e-4).  Up to 256 states -- one wave per
+    // SIMD, bound by latency more than by arithmetic -- double costs 7 % of the recursion and is used
+    // for sequences with fewer than four frames per state; beyond that it costs 15-20 % and is kept for
+    // sequences with fewer than five frames for every three states.  More than 4096 frames: always.
+    // The dense instance has no room in LDS.
+    const bool wide = !DENSE && ((cls == 1 && m.SP <= 256 && m.L < 4LL * m.S) || 5LL * m.S > 3LL * m.L || m.L > 4096);
     if (wide) {
         double* st0 = (double*)stf;
-        recurse_dispatch<SYNC, T_, double>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);
+        recurse_dispatch<SYNC, T_, double, true>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);
     } else {
-        recurse_dispatch<SYNC, T_, float>(a, m, b, dir, cls, stf, stf + (S_MAX + 16), amr[0], amr[1], wmin);
+        recurse_dispatch<SYNC, T_, float, true>(a, m, b, dir, cls, stf, stf + (S_MAX + 16), amr[0], amr[1], wmin);
     }
 }
 
@@ -1417,8 +1430,10 @@ __device__ __forceinline__ float slot_sum(const float* xs, const int c0, const i
     return s;
 }
 
+// (three waves per SIMD: with the headline workload's 48 KB row image three workgroups share a
+// compute unit, and the register count must not stand in the way)
 template <bool SYNC>
-__global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
+__global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
@@ -1615,6 +1630,67 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_combine(CombArgs a) {
                 sd[js] = slot_sum(xs, c0[js], c1[js]);
                 lsum += sd[js];
             }
+            const float tot = block_sum256(lsum, redsum);
+            finish_row(t, mn, tot, sd, em, JS, offs);
+        }
+    } else if (nE <= COMB_MID_EDGES && D <= COMB_MID_SLOTS) {
+        // medium sequences: this thread's edges still stay in registers for the whole strip (sixteen
+        // of them, source and target packed), the operands of a frame are fetched in one go, and the
+        // scores go through the LDS staging area in up to four passes
+        constexpr int JE = COMB_MID_EDGES / COMB_THREADS, JS = COMB_MID_SLOTS / COMB_THREADS, JP = COMB_XS / COMB_THREADS;
+        unsigned eft[JE], esl[JE];
+        float ew[JE];
+#pragma unroll
+        for (int j = 0; j < JE; j++) {
+            const int i = tid + j * COMB_THREADS;
+            uint4 r = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+            if (i < nE) r = crec[i];
+            eft[j] = r.x; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
+        }
+        int em[JS];
+#pragma unroll
+        for (int js = 0; js < JS; js++) {
+            const int d = tid + js * COMB_THREADS;
+            em[js] = d < D ? de[d] : 0;
+        }
+        const int npass = (nE + COMB_XS - 1) / COMB_XS;
+        for (int t = t0; t < tv; t++) {
+            const float* arow = abase + (size_t)t * SP;
+            const float* brow = bbase + (size_t)t * SP;
+            const float* grow = gbase + (size_t)t * DP;
+            float x[JE];
+            float lmin = INF_F;
+#pragma unroll
+            for (int j = 0; j < JE; j++) {
+                x[j] = (load_x<SYNC>(arow + (eft[j] & 0xFFFFu)) + ew[j]) + (load_x<SYNC>(grow + esl[j]) + load_x<SYNC>(brow + (eft[j] >> 16)));
+                lmin = fminf(lmin, x[j]);
+            }
+            const double offs = tid == 0 ? load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t) : 0.0;
+            const float mn = block_min256(lmin, redmin);
+            float sd[JS];
+#pragma unroll
+            for (int js = 0; js < JS; js++) sd[js] = 0.f;
+#pragma unroll
+            for (int p = 0; p < JE / JP; p++) {
+                if (p < npass) {
+                    const int p0 = p * COMB_XS, p1 = min(nE, p0 + COMB_XS);
+                    if (p > 0) __syncthreads();
+#pragma unroll
+                    for (int jj = 0; jj < JP; jj++)
+                        xs[tid + jj * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[p * JP + jj]);
+                    __syncthreads();
+#pragma unroll
+                    for (int js = 0; js < JS; js++) {
+                        const int d = tid + js * COMB_THREADS;
+                        int e0 = 0, e1 = 0;
+                        if (d < D) { e0 = max(cb[d], p0) - p0; e1 = min(cb[d + 1], p1) - p0; }
+                        sd[js] += slot_sum(xs, e0, e1);
+                    }
+                }
+            }
+            float lsum = 0.f;
+#pragma unroll
+            for (int js = 0; js < JS; js++) lsum += sd[js];
             const float tot = block_sum256(lsum, redsum);
             finish_row(t, mn, tot, sd, em, JS, offs);
         }
