@@ -1230,11 +1230,6 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
     // gather or combine waves
     __builtin_amdgcn_s_setprio(3);
-    // In the schedule in which gather and dense write run at the same time the workgroup also claims
-    // the registers that would let their waves move in beside its own: the nine waves then hold 504
-    // (one SIMD) or 336 of a SIMD's 512 registers, as much as three waves per SIMD allow.  Measured on
-    // the headline workload: with the 142 registers the code needs, 0.575 ms per call; with 168, 0.553.
-    if (SYNC && !DENSE) asm volatile("v_mov_b32 v167, 0" ::: "v167");
     if (SYNC) {
         // This kernel is started beside the preparation, so that its large workgroups are placed
         // while the machine is still empty: report the placement (see fbw_gate), wait until all
@@ -1291,9 +1286,17 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     }
 }
 
-template <bool SYNC>
+// RESERVE: in the schedule in which gather and dense write run at the same time the workgroup also
+// claims the registers that would let their waves move in beside its own: its nine waves then hold
+// 504 (one SIMD) or 336 of a SIMD's 512 registers, as much as three waves per SIMD allow.  Measured
+// on the headline workload: with the 142 registers the code needs, 0.575 ms per call; with 168,
+// 0.553.  Only for batches that leave half of the compute units without a recursion workgroup:
+// 256-thread workgroups need room on every SIMD, and with one of these on every unit the gather
+// would find none anywhere.
+template <bool SYNC, bool RESERVE = false>
 __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS_F64];
+    if (RESERVE) asm volatile("v_mov_b32 v167, 0" ::: "v167");
     recurse_workgroup<SYNC, false>(a, lds);
 }
 // The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS_F32 floats): with the
@@ -2074,7 +2077,8 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     const bool early = overlap && 2 * B <= P.n_cu / 2;
     auto launch_recursion = [&]() -> int {
         { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
-          else hipLaunchKernelGGL(fbw_recurse<true>, dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
+          else if (early) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
+          else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
         HIP_TRY(hipGetLastError());
         HIP_TRY(hipEventRecord(P.doneR, sR));
         return I6FBW_OK;

@@ -82,6 +82,9 @@ def test_tightly_constrained_alignment(oracle):
     ("cart", dict(T=40, B=2, F=38000, n_labels=(8, 12))),     # the largest row images that fit into LDS
     ("ctc", dict(T=40, B=8, F=50)),
     ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
+    ("cart", dict(T=60, B=64, F=300, n_labels=(5, 9))),      # a recursion workgroup on half of the compute units: started beside the preparation
+    ("cart", dict(T=60, B=65, F=300, n_labels=(5, 9))),      # one more: started behind it
+    ("cart", dict(T=60, B=128, F=300, n_labels=(5, 9))),     # one on every compute unit: gather and dense write must still find room
     ("ctc", dict(T=30, B=200, F=40)),          # 400 recursion workgroups: two per compute unit, started behind the preparation
     ("ctc", dict(T=30, B=256, F=40)),          # exactly two recursion workgroups on every compute unit
     ("ctc", dict(T=24, B=600, F=40)),          # more recursion workgroups than the device holds at once
