@@ -2013,7 +2013,12 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // By default only where it pays: a large dense tensor, and a batch whose recursion workgroups
     // leave wave slots free on every compute unit (with two of them on each unit the gather crawls:
     // T=200, B=256, F=5001 takes 0.49 ms overlapped against 0.40 ms stage after stage).
-    bool overlap = forced >= 0 ? forced != 0 : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu);
+    // Nor with few frames (there is little recursion to hide: up to 300 frames the stages in a row
+    // are as fast or up to 20 % faster at F = 12001) or, unless the sequences are long, with a handful
+    // of sequences (8 sequences of 1000 frames: 9 % slower overlapped; 8 of 4000 frames with large
+    // automata: 25 % faster).
+    bool overlap = forced >= 0 ? forced != 0
+                               : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu && T >= 384 && (B >= 12 || T >= 2048));
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
     if (2 * B > (T <= 4096 ? 2 : 1) * P.n_cu) overlap = false;
