@@ -1192,7 +1192,8 @@ constexpr int REC_LDS_FLOATS_F64 = 2 * D_MAX + 4 * (S_MAX + 16) + 32 + 8;
 // the compute threads' part for one state type; the loader waves do not depend on it
 // ONE: whether sequences with one state per thread can arrive here with this state type (they are
 // not instantiated otherwise: fewer loop bodies in a kernel give the remaining ones better code)
-template <bool SYNC, int T_, typename ST, bool ONE>
+// MANY: the same for the larger classes and the table-driven fallback
+template <bool SYNC, int T_, typename ST, bool ONE, bool MANY = true>
 __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int cls,
                                                  ST* st0, ST* st1, const float* am0, const float* am1, float* wmin) {
     const int K = dir ? m.Kout : m.Kin;
@@ -1200,7 +1201,7 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     // (No six-edge specialisation for double: it is the rare case.)
     constexpr bool F32 = sizeof(ST) == 4;
-    if (K > KMAX) {
+    if (MANY && K > KMAX) {
         recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
     } else if (ONE && cls == 1) {
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
@@ -1208,6 +1209,8 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (F32 && K <= 6) recurse_compute<SYNC, T_, 1, F32 ? 6 : KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute<SYNC, T_, 1, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+    } else if (!MANY) {
+        return;
     } else if (cls == 2) {
         if (K <= 2) recurse_compute<SYNC, T_, 4, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 4, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
@@ -1276,9 +1279,17 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // SIMD, bound by latency more than by arithmetic -- double costs 7 % of the recursion and is used
     // for sequences with fewer than four frames per state; beyond that it costs 15-20 % and is kept for
     // sequences with fewer than five frames for every three states.  More than 4096 frames: always.
-    // The dense instance has no room in LDS.
-    const bool wide = !DENSE && ((cls == 1 && m.SP <= 256 && m.L < 4LL * m.S) || 5LL * m.S > 3LL * m.L || m.L > 4096);
-    if (wide) {
+    // The dense instance has room in LDS for the small sequences only (and is used for at most 4096
+    // frames): batches of more than 128 CTC automata of 110-150 labels over 760-900 frames came out at
+    // 8.7e-5 to 9.3e-5 in float.
+    const bool small_tight = cls == 1 && m.SP <= 256 && m.L < 4LL * m.S;
+    const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > 4096);
+    // (there double costs half of the recursion time again, so only from 384 frames on, where the
+    // rounding of float has had time to add up; but for every sequence with one state per thread)
+    if (DENSE && cls == 1 && m.L < 4LL * m.S && m.L >= 384 && (dir ? m.Kout : m.Kin) <= KMAX) {
+        double* st0 = (double*)stf;
+        recurse_dispatch<SYNC, T_, double, true, false>(a, m, b, dir, cls, st0, st0 + (T_ + 16), amr[0], amr[1], wmin);
+    } else if (wide) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);
     } else {

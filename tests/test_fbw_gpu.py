@@ -175,3 +175,13 @@ def test_one_class_on_many_edges(oracle, n_labels):
     in registers, edges staged in passes)."""
     W = make_workload("ctc", T=3 * n_labels, B=2, F=n_labels + 200, n_labels=(n_labels, n_labels + 1))
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
+
+
+def test_large_batch_of_tightly_aligned_ctc(oracle):
+    """More than 128 sequences (the recursion instance of which two workgroups share a compute unit) of
+    CTC automata with 116 labels over up to 850 frames: float state vectors came out at 9e-5 here; the
+    small sequences of such batches keep theirs in double."""
+    W = make_workload("ctc", seed=2, T=850, B=140, F=300, n_labels=(116, 117))
+    out, loss = check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=16)
+    want_out, _ = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states, threads=16)
+    assert np.abs(posterior(out) - posterior(want_out)).max() < 4e-5
