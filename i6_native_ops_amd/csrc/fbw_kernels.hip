@@ -1278,15 +1278,17 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // 1055 frames 1.4e-4; 20 000 frames through 100 states 3e-4).  Up to 256 states -- one wave per
     // SIMD, bound by latency more than by arithmetic -- double costs 7 % of the recursion and is used
     // for sequences with fewer than four frames per state; beyond that it costs 15-20 % and is kept for
-    // sequences with fewer than five frames for every three states.  More than 4096 frames: always.
+    // sequences with fewer than five frames for every three states.  More than 1024 frames: always
+    // (whatever the shape of the automaton, float adds up to about 1e-4 over 2000 frames: CTC automata of
+    // 200 labels over 2000 frames 9.7e-5, of 400 labels over 2600 frames 8e-5).
     // The dense instance has room in LDS for the small sequences only (and is used for at most 4096
     // frames): batches of more than 128 CTC automata of 110-150 labels over 760-900 frames came out at
     // 8.7e-5 to 9.3e-5 in float.
     const bool small_tight = cls == 1 && m.SP <= 256 && m.L < 4LL * m.S;
-    const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > 4096);
+    const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > 1024);
     // (there double costs half of the recursion time again, so only from 384 frames on, where the
     // rounding of float has had time to add up; but for every sequence with one state per thread)
-    if (DENSE && cls == 1 && m.L < 4LL * m.S && m.L >= 384 && (dir ? m.Kout : m.Kin) <= KMAX) {
+    if (DENSE && cls == 1 && ((m.L < 4LL * m.S && m.L >= 384) || m.L > 1024) && (dir ? m.Kout : m.Kin) <= KMAX) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true, false>(a, m, b, dir, cls, st0, st0 + (T_ + 16), amr[0], amr[1], wmin);
     } else if (wide) {
