@@ -14,7 +14,7 @@ from tests.gpu_util import DeviceProblem
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("name", ["cart", "ctc", "longform"])
+@pytest.mark.parametrize("name", ["cart", "monophone", "ctc", "longform"])
 def test_full_size(oracle, name):
     W = make_workload(name)
     print(f"full size {name}: T={W.T} B={W.B} F={W.F} E={W.E}", flush=True)
@@ -47,6 +47,7 @@ def test_full_size(oracle, name):
     for t0 in range(0, W.T, 100):                       # in slices: exp() of the whole tensor at once is 12 GB in float64
         ref = np.exp(-want_out[t0:t0 + 100].astype(np.float64))
         worst = max(worst, float(np.abs(got[t0:t0 + 100] - ref).max()))
+    print(f"full size {name}: worst posterior error {worst:.1e}", flush=True)
     assert worst <= 1e-4
     del got, want_out
 
