@@ -21,7 +21,10 @@ SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read
            "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment", "i6fbw_set_band",
            "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
            "i6fbw_profile_enable", "i6fbw_profile_read",
-           "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode")
+           "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode",
+           "i6fbw_run_static", "i6fbw_static_workspace")
+STATIC_WORKSPACE_BYTES = 32 << 20
+ERR_STATIC_WORKSPACE = -16
 
 _lib = None
 
@@ -44,6 +47,12 @@ def load():
                                           c.c_int, c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t,
                                           c.c_void_p]
         lib.i6fbw_run_strided.restype = c.c_int
+        lib.i6fbw_run_static.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_int64, c.c_void_p, c.c_void_p,
+                                         c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
+                                         c.c_void_p, c.c_void_p, c.c_void_p]
+        lib.i6fbw_run_static.restype = c.c_int
+        lib.i6fbw_static_workspace.argtypes = [c.POINTER(c.c_void_p), c.POINTER(c.c_size_t)]
+        lib.i6fbw_static_workspace.restype = c.c_int
         lib.i6fbw_viterbi.argtypes = [c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_int64, c.c_void_p, c.c_void_p,
                                       c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int,
                                       c.c_void_p, c.c_int64, c.c_int64, c.c_void_p, c.c_void_p, c.c_size_t, c.c_void_p]
@@ -111,6 +120,24 @@ def run(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_pt
                           ws_bytes, stream)
     if rc != 0:
         raise FbwError(rc)
+
+
+def run_static(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr, se_row_stride,
+               seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, sum_ptr, stream=0) -> None:
+    """i6fbw_run in the library's built-in workspace: allocates nothing."""
+    rc = load().i6fbw_run_static(am_ptr, am_stride_t, am_stride_b, edges_ptr, edge_row_stride, weights_ptr, start_end_ptr,
+                                 se_row_stride, seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, sum_ptr, stream)
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def static_workspace():
+    """(device address, bytes) of the current device's built-in workspace."""
+    ptr, n = ctypes.c_void_p(0), ctypes.c_size_t(0)
+    rc = load().i6fbw_static_workspace(ctypes.byref(ptr), ctypes.byref(n))
+    if rc != 0:
+        raise FbwError(rc)
+    return int(ptr.value), int(n.value)
 
 
 def run_strided(am_ptr, am_stride_t, am_stride_b, scores_are_log_probs, edges_ptr, edge_row_stride, weights_ptr,

@@ -29,6 +29,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <mutex>
@@ -1828,7 +1829,9 @@ thread_local hipError_t g_last_hip_error = hipSuccess;
 // beside them on two streams of its own; the kernels that run at the same time feed each other
 // through flags in memory.
 struct Pipeline {
-    bool ready = false;
+    std::mutex mu;            // calls on one device are serialised (they share its streams and events); devices are independent
+    bool attr_ready = false;  // kernel attributes set, device facts read
+    bool ready = false;       // streams and events created
     hipStream_t sP = nullptr, sR = nullptr;
     hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneR = nullptr;
     int n_cu = 256;
@@ -1836,9 +1839,15 @@ struct Pipeline {
     // caller streams that were checked against the recursion stream: do kernels on the two run at
     // the same time?
     std::vector<std::pair<hipStream_t, bool>> checked;
+    void* static_ws = nullptr;   // this device's copy of g_static_workspace (i6fbw_run_static)
 };
 Pipeline g_pipe[MAX_DEVICES];
-std::mutex g_mutex;
+std::mutex g_mutex;           // process-wide settings and the stage profile
+
+// Built-in workspace of i6fbw_run_static, for callers that cannot allocate device memory.  Every
+// device the library runs on holds its own copy for the life of the process; host code reaches it
+// only through the address hipGetSymbolAddress returns for the current device (Pipeline::static_ws).
+static __device__ __align__(256) unsigned char g_static_workspace[I6FBW_STATIC_WORKSPACE_BYTES];
 
 // LDS of a preparation workgroup: sort keys, emission bitmap and its prefix counts
 size_t prep_lds_bytes(int F) { return (size_t)EB_MAX * 4 + (F <= F_BITMAP_MAX ? (size_t)((F + 31) >> 5) * 8 : 0); }
@@ -1851,16 +1860,12 @@ void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
     else hipLaunchKernelGGL(fbw_prepare<1024>, dim3(3, pa.B), dim3(1024), lds, s, pa);
 }
 
-int pipeline_init(Pipeline& p) {
-    if (p.ready) return I6FBW_OK;
+// Device facts and kernel attributes; creates nothing (i6fbw_run_static stops here).
+int device_init(Pipeline& p) {
+    if (p.attr_ready) return I6FBW_OK;
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     HIP_TRY(hipDeviceGetAttribute(&p.n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    // default priority on purpose
-    HIP_TRY(hipStreamCreateWithFlags(&p.sP, hipStreamNonBlocking));
-    HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
-    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
-        HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
@@ -1870,6 +1875,20 @@ int pipeline_init(Pipeline& p) {
     hipFuncAttributes attr;
     HIP_TRY(hipFuncGetAttributes(&attr, (const void*)fbw_recurse_dense<true>));
     p.dense_regs = attr.numRegs;
+    // address of the current device's copy of the built-in workspace
+    HIP_TRY(hipGetSymbolAddress(&p.static_ws, HIP_SYMBOL(g_static_workspace)));
+    p.attr_ready = true;
+    return I6FBW_OK;
+}
+
+int pipeline_init(Pipeline& p) {
+    if (p.ready) return I6FBW_OK;
+    { int rc = device_init(p); if (rc != I6FBW_OK) return rc; }
+    // default priority on purpose
+    HIP_TRY(hipStreamCreateWithFlags(&p.sP, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
+    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
+        HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     p.ready = true;
     return I6FBW_OK;
 }
@@ -1898,7 +1917,7 @@ int runs_beside(Pipeline& p, hipStream_t s, bool* yes) {
 
 // Stage timing: event pairs around every launch of a stage, on the stream it runs on.
 struct Profile {
-    bool on = false;
+    std::atomic<bool> on{false};
     static constexpr int MAXPAIR = 8192;
     int n_pairs = 0, n_calls = 0;
     hipEvent_t a[MAXPAIR], b[MAXPAIR];
@@ -1910,8 +1929,10 @@ Profile g_prof;
 struct StageTimer {
     int idx = -1;
     hipStream_t stream;
-    StageTimer(int stage, hipStream_t st) : stream(st) {
-        if (!g_prof.on || g_prof.n_pairs >= Profile::MAXPAIR) return;
+    StageTimer(int stage, hipStream_t st, bool enabled) : stream(st) {
+        if (!enabled) return;
+        std::lock_guard<std::mutex> lock(g_mutex);      // the profile is shared by all devices
+        if (g_prof.n_pairs >= Profile::MAXPAIR) return;
         if (g_prof.n_pairs >= g_prof.n_created) {
             if (hipEventCreate(&g_prof.a[g_prof.n_created]) != hipSuccess) return;
             if (hipEventCreate(&g_prof.b[g_prof.n_created]) != hipSuccess) return;
@@ -1930,11 +1951,11 @@ size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size
 constexpr int COMB_TILE_W = 12288;     // floats of a row that go through LDS at a time when the row does not fit: three workgroups per unit
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
-int g_no_band = 0;      // see i6fbw_set_band
-int g_overlap_mode = [] {
+std::atomic<int> g_no_band{0};      // see i6fbw_set_band
+std::atomic<int> g_overlap_mode{[] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
-}();
+}()};
 
 // Status reports that travel to the host without a wait: per device a ring of pinned {code, seq}
 // slots, each with the event that follows its copy on the caller's stream.
@@ -1962,12 +1983,18 @@ bool status_collect(StatusRing& r, int i, bool wait) {
 
 // how the bindings report device-side problems: 0 not at all, 1 by waiting for every call, 2 without
 // waiting, at a later call; I6FBW_STATUS=off|sync|deferred sets the initial value (I6FBW_ASYNC=1: off)
-int g_status_mode = [] {
+std::atomic<int> g_status_mode{[] {
     const char* e = getenv("I6FBW_STATUS");
     if (e) return e[0] == 'o' ? 0 : (e[0] == 's' ? 1 : 2);
     const char* a = getenv("I6FBW_ASYNC");
     return (a && a[0] == '1') ? 0 : 2;
-}();
+}()};
+
+int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+             const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
+             int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
+             int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
+             void* workspace, size_t workspace_bytes, void* stream_, const bool static_call);
 
 }  // namespace
 
@@ -1993,15 +2020,53 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
                       int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
                       int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
                       void* workspace, size_t workspace_bytes, void* stream_) {
+    return run_impl(am, am_stride_t, am_stride_b, scores_are_log_probs, edges, edge_row_stride, weights, start_end,
+                    se_row_stride, seq_lens, T, B, F, E, n_states, out_mode, out, out_stride_t, out_stride_b, sum_output,
+                    workspace, workspace_bytes, stream_, false);
+}
+
+int i6fbw_run_static(const float* am, int64_t am_stride_t, int64_t am_stride_b, const int32_t* edges, int64_t edge_row_stride,
+                     const float* weights, const int32_t* start_end, int64_t se_row_stride, const int32_t* seq_lens, int T,
+                     int B, int F, int E, int n_states, int out_mode, float* out, float* sum_output, void* stream_) {
+    // workspace == nullptr: run_impl takes the current device's built-in buffer
+    return run_impl(am, am_stride_t, am_stride_b, 0, edges, edge_row_stride, weights, start_end, se_row_stride, seq_lens,
+                    T, B, F, E, n_states, out_mode, out, (int64_t)B * F, (int64_t)F, sum_output, nullptr, 0, stream_, true);
+}
+
+int i6fbw_static_workspace(void** workspace, size_t* bytes) {
+    if (!workspace || !bytes) return I6FBW_ERR_INVALID_ARGUMENT;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
+    Pipeline& P = g_pipe[dev];
+    std::lock_guard<std::mutex> lock(P.mu);
+    { int rc = device_init(P); if (rc != I6FBW_OK) return rc; }
+    *workspace = P.static_ws; *bytes = I6FBW_STATIC_WORKSPACE_BYTES;
+    return I6FBW_OK;
+}
+
+}  // extern "C"
+
+namespace {
+// Body of i6fbw_run_strided and i6fbw_run_static.  static_call: the workspace is the device's
+// built-in buffer, and nothing may be allocated or created -- no library streams or events, no
+// stage timers: the stages run one after the other on the caller's stream.
+int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+             const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
+             int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
+             int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
+             void* workspace, size_t workspace_bytes, void* stream_, const bool static_call) {
     if (T <= 0 || B <= 0 || F <= 0 || E < 0 || n_states <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
-    if (!am || !start_end || !seq_lens || !out || !sum_output || !workspace) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (!am || !start_end || !seq_lens || !out || !sum_output || (!workspace && !static_call)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (E > 0 && (!edges || !weights)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB && out_mode != I6FBW_OUT_NEG_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_stride_t < 0 || out_stride_b < 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
     const Layout l = make_layout(T, B, E);
-    if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
+    if (static_call) {
+        if (l.total > (size_t)I6FBW_STATIC_WORKSPACE_BYTES) return I6FBW_ERR_STATIC_WORKSPACE;
+    } else if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
     // too many emission classes for the LDS bitmap of the preparation: every sequence takes the general path
     const bool f_too_large = F > F_BITMAP_MAX;
     // rows too long for the LDS image of the dense write go through it in tiles; so do rows of more
@@ -2013,16 +2078,17 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
-    std::lock_guard<std::mutex> lock(g_mutex);
     Pipeline& P = g_pipe[dev];
-    { int rc = pipeline_init(P); if (rc != I6FBW_OK) return rc; }
+    std::lock_guard<std::mutex> lock(P.mu);
+    { int rc = static_call ? device_init(P) : pipeline_init(P); if (rc != I6FBW_OK) return rc; }
+    if (static_call) workspace = P.static_ws;
 
     hipStream_t s = (hipStream_t)stream_;
     char* ws = (char*)workspace;
     SeqMeta* meta = (SeqMeta*)(ws + l.meta);
     int* sync = (int*)(ws + l.sync);
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
-    const int forced = g_overlap_mode;
+    const int forced = static_call ? 0 : g_overlap_mode.load();
     // By default only where it pays: a large dense tensor, and a batch whose recursion workgroups
     // leave wave slots free on every compute unit (with two of them on each unit the gather crawls:
     // T=200, B=256, F=5001 takes 0.49 ms overlapped against 0.40 ms stage after stage).
@@ -2046,7 +2112,8 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     }
     if (overlap) { int rc = runs_beside(P, s, &overlap); if (rc != I6FBW_OK) return rc; }
     hipStream_t sP = overlap ? P.sP : s, sR = overlap ? P.sR : s;
-    if (g_prof.on) g_prof.n_calls++;
+    const bool timed = g_prof.on && !static_call;     // stage timers create events
+    if (timed) { std::lock_guard<std::mutex> plock(g_mutex); g_prof.n_calls++; }
 
     const dim3 g_grid((unsigned)B * ((T + TG - 1) / TG)), c_grid((unsigned)B * ((T + TC - 1) / TC));
     const dim3 p_grid(B, (T + TC - 1) / TC);
@@ -2084,7 +2151,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
 
     {
         // the scan also clears the header of the hand-off area, so it runs even without edges
-        StageTimer tm(0, s);
+        StageTimer tm(0, s, timed);
         hipLaunchKernelGGL(fbw_scan_sorted, dim3(std::max(1, (E + SCAN_BLOCK - 1) / SCAN_BLOCK)), dim3(256), 0, s,
                            E > 0 ? edges + 3 * edge_row_stride : nullptr, E, B, pa.sortflag, pa.seqbegin, sync);
         HIP_TRY(hipGetLastError());
@@ -2094,7 +2161,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // LDS and could otherwise find no room while the recursion waits for them), else behind it.
     const bool early = overlap && 2 * B <= P.n_cu / 2;
     auto launch_recursion = [&]() -> int {
-        { StageTimer tm(2, sR); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
+        { StageTimer tm(2, sR, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
           else if (early) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
           else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
         HIP_TRY(hipGetLastError());
@@ -2115,7 +2182,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
         }
     }
     {
-        StageTimer tm(0, s);
+        StageTimer tm(0, s, timed);
         launch_prepare(P, pa, s);
         HIP_TRY(hipGetLastError());
     }
@@ -2127,7 +2194,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
     // leaves the memory system idle.
     {
-        StageTimer tm(4, sP);
+        StageTimer tm(4, sP, timed);
         hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
                            (long long)out_stride_b, sum_output);
         HIP_TRY(hipGetLastError());
@@ -2135,12 +2202,12 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     if (overlap) HIP_TRY(hipEventRecord(P.doneP, sP));
 
     if (!overlap) {
-        { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
+        { StageTimer tm(1, s, timed); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(2, s); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, s, ra);
+        { StageTimer tm(2, s, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, s, ra);
           else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+        { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
         HIP_TRY(hipGetLastError());
         return I6FBW_OK;
     }
@@ -2150,7 +2217,7 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
     // held back until every recursion workgroup is on the machine -- normally long since.
     hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
     HIP_TRY(hipGetLastError());
-    { StageTimer tm(1, s); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, s, ga); }
+    { StageTimer tm(1, s, timed); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, s, ga); }
     HIP_TRY(hipGetLastError());
     // The dense write follows the gather on the same stream (its workgroups would only take wave
     // slots away from the gather before that: by then the two recursions are about to meet in the
@@ -2159,13 +2226,16 @@ int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b,
 #ifdef I6_TRACE
     if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
 #endif
-    { StageTimer tm(3, s); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+    { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
     HIP_TRY(hipGetLastError());
     // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     return I6FBW_OK;
 }
+}  // namespace
+
+extern "C" {
 
 // a stream that is being captured into a graph can neither be waited for nor carry the events of
 // the status ring: no report from there
@@ -2204,7 +2274,7 @@ int i6fbw_post_status(void* workspace, int B, void* stream) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_pipe[dev].mu);
     StatusRing& r = g_status[dev];
     if (!r.host) HIP_TRY(hipHostMalloc((void**)&r.host, sizeof(int) * 2 * StatusRing::SLOTS, hipHostMallocDefault));
     const int i = r.next;
@@ -2229,7 +2299,7 @@ int i6fbw_poll_status(int wait, int* code, int* seq) {
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
-    std::lock_guard<std::mutex> lock(g_mutex);
+    std::lock_guard<std::mutex> lock(g_pipe[dev].mu);
     StatusRing& r = g_status[dev];
     // oldest first; reports arrive in the order of the calls (on one stream), so the first one that
     // is still on its way ends the search: a poll costs one or two event queries, not sixty-four
@@ -2263,6 +2333,7 @@ const char* i6fbw_strerror(int code) {
         case I6FBW_ERR_SEQ_TOO_LARGE: return "a sequence has more than 4096 states or distinct emissions";
         case I6FBW_ERR_BAD_INDEX: return "sequence, emission or state index out of range";
         case I6FBW_ERR_TIMEOUT: return "a kernel gave up waiting for another stage of the same call";
+        case I6FBW_ERR_STATIC_WORKSPACE: return "the problem needs more workspace than the built-in buffer of i6fbw_run_static holds (32 MiB)";
         default: return "unknown status";
     }
 }

@@ -39,7 +39,8 @@ enum {
                                              general path do not fit its share of the workspace (T < 2*edges+16 with
                                              state ids spread over nearly 2*edges ids) */
     I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
-    I6FBW_ERR_TIMEOUT = -15               /* device-side: a stage gave up waiting for another stage of the call */
+    I6FBW_ERR_TIMEOUT = -15,              /* device-side: a stage gave up waiting for another stage of the call */
+    I6FBW_ERR_STATIC_WORKSPACE = -16      /* i6fbw_run_static: the problem needs more than I6FBW_STATIC_WORKSPACE_BYTES */
 };
 
 /* Layout of the posterior tensor written by i6fbw_run. */
@@ -116,6 +117,30 @@ int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_st
                       int T, int B, int F, int E, int n_states, int out_mode,
                       float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * i6fbw_run for callers that cannot allocate device memory and therefore have no workspace to
+ * bring: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference (whose fbw_cuda allocates and frees three buffers per call,
+ * fbw_op.cu:283-286,384-386).  Same arguments and results as i6fbw_run without the workspace: the
+ * kernels work in a built-in device buffer of I6FBW_STATIC_WORKSPACE_BYTES that every GPU the
+ * library runs on holds until the process ends.  The call allocates nothing (no device or host
+ * memory, no streams, no events) and runs all stages one after the other on `stream`.
+ * Problems whose workspace (i6fbw_workspace_size) is larger than the built-in buffer are refused
+ * with I6FBW_ERR_STATIC_WORKSPACE.  All calls on one GPU share the one buffer: calls that overlap
+ * in time on the same GPU (two streams, two host threads) race; calls on one stream are ordered
+ * and safe.  i6fbw_static_workspace hands out the buffer of the current device, e.g. for
+ * i6fbw_read_status(buffer, B, stream, ...) after a call.
+ */
+#define I6FBW_STATIC_WORKSPACE_BYTES (32u << 20)
+int i6fbw_run_static(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
+                     const int32_t* edges, int64_t edge_row_stride,
+                     const float* weights,
+                     const int32_t* start_end, int64_t se_row_stride,
+                     const int32_t* seq_lens,
+                     int T, int B, int F, int E, int n_states, int out_mode,
+                     float* out, float* sum_output, void* stream);
+int i6fbw_static_workspace(void** workspace, size_t* bytes);
 
 /*
  * Waits for `stream` and copies the device-side status of the last i6fbw_run that

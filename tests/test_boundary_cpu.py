@@ -83,3 +83,12 @@ def test_workload_generators_are_deterministic_and_well_formed():
     assert (w.T, w.B, w.F) == (1000, 32, 12001)
     per_seq_states = np.diff(np.append(w.start_end_states[0], w.n_states))
     assert per_seq_states.max() <= 451 and per_seq_states.min() >= 301
+
+
+def test_static_entry_point_refuses_large_problems_on_the_host():
+    """i6fbw_run_static checks the size against its built-in workspace before it touches the device."""
+    from i6_native_ops_amd import cabi
+    import pytest
+    with pytest.raises(cabi.FbwError) as e:
+        cabi.run_static(256, 32 * 12001, 12001, 256, 30000, 256, 256, 32, 256, 1000, 32, 12001, 30000, 12000, 0, 256, 256, 0)
+    assert e.value.code == cabi.ERR_STATIC_WORKSPACE
