@@ -22,7 +22,7 @@ SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read
            "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
            "i6fbw_profile_enable", "i6fbw_profile_read",
            "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode",
-           "i6fbw_run_static", "i6fbw_static_workspace")
+           "i6fbw_run_static", "i6fbw_static_workspace", "i6fbw_set_dense_writer")
 STATIC_WORKSPACE_BYTES = 32 << 20
 ERR_STATIC_WORKSPACE = -16
 
@@ -89,6 +89,8 @@ def load():
         lib.i6fbw_last_hip_error.restype = c.c_char_p
         lib.i6fbw_set_overlap.argtypes = [c.c_int]
         lib.i6fbw_set_overlap.restype = None
+        lib.i6fbw_set_dense_writer.argtypes = [c.c_int]
+        lib.i6fbw_set_dense_writer.restype = None
         lib.i6fbw_profile_enable.argtypes = [c.c_int]
         lib.i6fbw_profile_enable.restype = None
         lib.i6fbw_profile_read.argtypes = [c.POINTER(c.c_float)]
@@ -188,6 +190,11 @@ def poll_status(wait=False):
 def set_overlap(mode: int) -> None:
     """-1: by problem size, 0: single stream, 1: overlapped stages."""
     load().i6fbw_set_overlap(int(mode))
+
+
+def set_dense_writer(mode: int) -> None:
+    """-1: by problem, 0: row by row, 1: flat spans wherever the output layout allows it."""
+    load().i6fbw_set_dense_writer(int(mode))
 
 
 def ctc_fsa_bounds(B, Lmax):

@@ -56,6 +56,11 @@ constexpr int TG = I6_TG;             // frames per gather workgroup
 #define I6_TC 8
 #endif
 constexpr int TC = I6_TC;             // frames per combine workgroup
+#ifndef I6_FLAT_TCF
+#define I6_FLAT_TCF 2
+#endif
+constexpr int FLAT_TCF = I6_FLAT_TCF; // frames per posterior job of the flat dense write (one flag each)
+static_assert(TC % FLAT_TCF == 0, "posterior jobs tile a strip");
 constexpr int RENORM = 8;             // frames between renormalisations of the state vector
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
@@ -74,7 +79,8 @@ constexpr unsigned NO_STATE = 0xFFFFu;
 constexpr int SEQ_GENERIC = 1;        // value of SeqMeta::err / errA / errB that routes a sequence to the general path
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
 constexpr int SYNC_HDR = 16;          // ints before the progress counters in the hand-off area:
-                                      // [0] abort flag, [1] recursion workgroups placed so far, [3] preparation workgroups finished
+                                      // [0] abort flag, [1] recursion workgroups placed so far, [3] preparation workgroups finished,
+                                      // [4..5] status report {code, sequence}, [6] longest sequence of the batch in frames
 constexpr int PUBLISH = 32;           // recursion steps between progress publications
 constexpr int SPIN_LIMIT = 1 << 20;   // polls before a waiting wave gives up
 // Scores are kept in units of log 2 inside the workspace (exp2/log2 are single instructions).
@@ -106,14 +112,16 @@ __device__ __forceinline__ unsigned renum_capacity(int n_edges) { return 2u * (2
 __device__ __forceinline__ unsigned renum_home(int id, unsigned cap) { return __umulhi((unsigned)id * 2654435761u, cap); }
 
 struct Layout {
-    size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, renum, offA, offB, alpha, beta, gtab, total;
+    size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, renum, cflag, wpfx, offA, offB, alpha, beta, gtab, total;
     long long ss_total, gg_total;
+    int wpfx_stride;      // ints per sequence in the emission rank table (0: F too large for it)
 };
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-Layout make_layout(long long T, long long B, long long E) {
+Layout make_layout(long long T, long long B, long long E, long long F = 1) {
     Layout l;
+    l.wpfx_stride = F <= F_BITMAP_MAX ? (int)(((F + 31) >> 5) + 2) : 0;
     l.ss_total = round16(2 * E) + 32 * B + 16;
     l.gg_total = round16(E) + 32 * B + 16;
     size_t o = 0;
@@ -134,6 +142,9 @@ Layout make_layout(long long T, long long B, long long E) {
     l.alpha = o;    o = align256(o + sizeof(float) * l.ss_total * T);
     l.beta = o;     o = align256(o + sizeof(float) * l.ss_total * T);
     l.gtab = o;     o = align256(o + sizeof(float) * l.gg_total * T);
+    // (behind everything else: the offsets above do not depend on F)
+    l.cflag = o;    o = align256(o + sizeof(int) * B * ((T + FLAT_TCF - 1) / FLAT_TCF));
+    l.wpfx = o;     o = align256(o + sizeof(int) * B * l.wpfx_stride);
     l.total = o;
     return l;
 }
@@ -248,6 +259,9 @@ struct PrepArgs {
     int force_generic;  // F is too large for the emission bitmap: every sequence takes the general path
     int2* renum;        // renumbering tables, two entries per state of room (see local_state)
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
+    int* cflag = nullptr;   // per (sequence, strip of TC frames): compact posteriors written (flat dense write); may be null
+    int* wpfx = nullptr;    // per sequence: number of distinct emissions below 32 * w, for w = 0 .. ceil(F / 32); may be null
+    int wpfx_stride = 0;
 };
 
 // sortflag[blk] = 1 if the sequence indices of edges [blk*SCAN_BLOCK, (blk+1)*SCAN_BLOCK] never
@@ -511,6 +525,12 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         for (int w = w0; w < w1; w++) { wordpfx[w] = run; run += __popc(bitmap[w]); }
         __syncthreads();
         if (D > D_MAX) generic = 1;
+        if (role == 2 && a.wpfx) {
+            // the rank table also goes to memory: the flat dense write finds with it the slots whose
+            // emission falls into a piece of a row
+            int* wp = a.wpfx + (size_t)b * a.wpfx_stride;
+            for (int w = tid; w < nwords + 2; w += NT) wp[w] = w < nwords ? wordpfx[w] : D;
+        }
     }
     const int DP = (int)round16(D > 0 ? D : 1);
 
@@ -566,6 +586,12 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         if (tid < 2) a.sync[SYNC_HDR + 2 * b + tid] = 0;
         int* gf = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * nstrip;
         for (int i = tid; i < nstrip; i += NT) gf[i] = 0;
+        if (a.cflag) {
+            const int ncf = (a.T + FLAT_TCF - 1) / FLAT_TCF;
+            int* cf = a.cflag + (size_t)b * ncf;
+            for (int i = tid; i < ncf; i += NT) cf[i] = 0;
+        }
+        if (tid == 0) atomicMax(&a.sync[6], L);      // longest sequence of the batch (header cleared by the scan kernel)
     }
     if (role == 2 && tid == 0) {
         SeqMeta* m = a.meta + b;
@@ -1336,10 +1362,24 @@ struct CombArgs {
     long long ost_t, ost_b;      // element strides of out over frames and sequences
     int* sync;
     int tile_w;                  // 0: the row image holds the whole row; else its width in floats (a multiple of 32), see finish_row
+    int direct_only;             // beside fbw_flat: only the sequences that kernel leaves to this one (flat_direct)
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 typedef float float4a __attribute__((ext_vector_type(4)));
+
+// Which kernel writes the rows t < seq_len of a sequence when the dense tensor goes out in flat
+// spans (fbw_flat): that kernel itself for sequences small enough for its register-resident
+// posterior jobs, fbw_combine (row by row, started beside it with direct_only set) for the larger
+// ones and for those on the general path.  Sequences with a reported problem or without edges have
+// constant rows, which the write jobs of fbw_flat produce by themselves.
+constexpr int COMB_FAST_EDGES = 1024, COMB_FAST_SLOTS = 512;
+__device__ __forceinline__ bool flat_fast(const SeqMeta& m) {
+    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= COMB_FAST_EDGES && m.D <= COMB_FAST_SLOTS;
+}
+__device__ __forceinline__ bool flat_direct(const SeqMeta& m) {
+    return seq_error(m) >= 0 && m.n_edges > 0 && m.L > 0 && !flat_fast(m);
+}
 
 // Row streaming.  Rows start at arbitrary 4-byte offsets (F need not be a multiple of 32), so the
 // row is addressed from the 128-byte line boundary below its start: chunk c covers floats
@@ -1463,6 +1503,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     strip_index(a.B, &b, &y);
     const SeqMeta m = a.meta[b];
     if (m.L == 0) return;                                      // fbw_padfill has written every row
+    if (a.direct_only && !flat_direct(m)) return;
     const int T = a.T, B = a.B, F = a.F;
     // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
     // forward and the backward recursion meet, so those rows are complete first
@@ -1501,7 +1542,14 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             s_ok = ok;
         }
         __syncthreads();
-        if (!s_ok) return;       // timed out: reported through the abort flag
+        if (!s_ok) {
+            // timed out (reported through the abort flag): the rows say so too
+            for (int t = t0; t < tv; t++) {
+                stream_const_row(a.out + t * a.ost_t + b * a.ost_b, a.F, __builtin_nanf(""));
+                if (tid == 0) a.sum_output[(size_t)t * a.B + b] = __builtin_nanf("");
+            }
+            return;
+        }
     }
     if (seq_error(m) > 0) {
         __shared__ float gred[32];
@@ -1756,6 +1804,426 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// stage 4, flat form (fbw_flat).  The dense tensor is mostly holes: of the 12001 floats of a row of
+// the headline workload about 370 carry a posterior.  Here the posteriors of a frame are first
+// computed in compact form (one float per distinct emission of the sequence), and the tensor is
+// then written as a flat sequence of 128-byte-aligned spans of FLAT_W floats, whatever the row
+// length: a span is built in LDS from the (at most two) compact rows it cuts and leaves as two
+// aligned 16-byte stores per thread.
+//
+// One kernel holds both kinds of job, in one dispatch order:
+//   posterior job (sequence b, FLAT_TCF frames): waits for the two recursions to have passed its
+//       frames, computes edge scores, frame normaliser and per-emission sums as fbw_combine does,
+//       writes loss and compact posteriors and raises the flag of its frames;
+//   write job (group, j): FLAT_KMAX spans of the group's rows; waits for the flags of the rows they
+//       cut.  A group is a strip of TC frames of all sequences (layout (T,B,F)) or of one sequence
+//       (layout (B,T,F)), i.e. a contiguous piece of the tensor, clipped to whole rows: lines cut
+//       by the ends of a group are shared with the neighbouring group and written element by
+//       element by both.
+// Strips are taken from the middle outwards (where the recursions meet), posterior jobs FLAT_AHEAD
+// strips ahead of the write jobs that need them.  Workgroups are dispatched in index order and a
+// job only ever waits for jobs with a smaller index (and for the recursion, which is resident before
+// this kernel starts), so the job that is waited for is running or done: no wait can block the
+// kernel, whatever the occupancy.
+//
+// Measured on the headline tensor (1.54 GB): a bare writer of this shape reaches 6.9 TB/s with two
+// workgroups per compute unit and 5.9 with eight -- more stores on their way than the memory
+// system takes at a time cost bandwidth -- but a write job spends most of its life waiting for
+// what it reads (two dependent rounds of 2-3 us under this load), which takes all eight to hide;
+// this kernel writes the tensor in 0.265 ms when it has the machine to itself (5.8 TB/s, 0.30 ms
+// for fbw_combine + fbw_padfill) and in 0.26 ms of work beside the recursion.
+// ---------------------------------------------------------------------------------------------
+constexpr int FLAT_W = 2048;                  // floats per span: two 16-byte stores per thread
+#ifndef I6_FLAT_AHEAD
+#define I6_FLAT_AHEAD 4
+#endif
+#ifndef I6_FLAT_KMAX
+#define I6_FLAT_KMAX 8
+#endif
+#ifndef I6_FLAT_OCC
+#define I6_FLAT_OCC 8
+#endif
+constexpr int FLAT_AHEAD = I6_FLAT_AHEAD;     // strips by which posterior jobs run ahead of the write jobs that need them
+constexpr int FLAT_KMAX = I6_FLAT_KMAX;       // spans per write job
+constexpr int FLAT_MIN_F = FLAT_W;            // a span then cuts at most two rows
+constexpr unsigned FLAT_SKIP = 0x7fc0deadu;   // image marker, a NaN no computation produces: element not written by this job
+
+struct FlatArgs {
+    CombArgs c;
+    int layout;            // 0: out is (T, B, F) contiguous, 1: (B, T, F) contiguous
+    int nW;                // write jobs per group
+    int K;                 // spans per write job
+    int shift;             // floats between the 128-byte line boundary below out and out
+    int* cflag;            // per (sequence, strip): 1 compact posteriors written, 2 given up
+    const int* wpfx; int wpfx_stride;
+    float* cp;             // compact posteriors [seq][t][slot], in the memory of the compact emission table:
+                           // row t of that table is last read by the posterior job that then overwrites it
+};
+
+// i-th strip of n in the order middle, middle+1, middle-1, middle+2, ... (the side that runs out first is skipped)
+__device__ __forceinline__ int middle_out(const int i, const int n, const int mid) {
+    const int up = n - 1 - mid, down = mid;
+    if (i <= 2 * min(up, down)) return (i & 1) ? mid + (i + 1) / 2 : mid - i / 2;
+    return up > down ? mid + (i - down) : mid - (i - up);
+}
+
+template <bool SYNC>
+__device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const int t0, float* xs, float* redmin, float* redsum,
+                                          int* s_ok) {
+    const CombArgs& a = fa.c;
+    const int tid = threadIdx.x;
+    const SeqMeta m = a.meta[b];
+    const int T = a.T, B = a.B;
+    const int t1 = min(T, t0 + FLAT_TCF);
+    if (t0 >= T) return;
+    const int L = m.L;
+    // frames from seq_len on: loss 0 (fbw_op.cu:120-128); their rows are holes, written by the write jobs
+    for (int t = max(t0, L) + tid; t < t1; t += COMB_THREADS) a.sum_output[(size_t)t * B + b] = 0.f;
+    const int tv = min(L, t1);
+    if (t0 >= tv) return;
+    const int err = seq_error(m);
+    if (err < 0 || m.n_edges == 0) {
+        for (int t = t0 + tid; t < tv; t += COMB_THREADS) a.sum_output[(size_t)t * B + b] = err < 0 ? __builtin_nanf("") : 0.f;
+        return;
+    }
+    if (!flat_fast(m)) return;              // fbw_combine writes loss and rows of this sequence
+    int* flag = fa.cflag + (size_t)b * ((T + FLAT_TCF - 1) / FLAT_TCF) + t0 / FLAT_TCF;
+    if (SYNC) {
+        if (tid == 0) {
+            const int* prog = a.sync + SYNC_HDR + 2 * b;
+            const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((a.T + TG - 1) / TG);
+            bool ok = true;
+            for (int g = t0 / TG; ok && g <= (tv - 1) / TG; g++) ok = spin_until_ge(gflag + g, 1, a.sync);
+            ok = ok && spin_until_ge(prog, tv, a.sync) && spin_until_ge(prog + 1, m.L - t0, a.sync);
+            *s_ok = ok;
+        }
+        __syncthreads();
+        if (!*s_ok) {
+            for (int t = t0 + tid; t < tv; t += COMB_THREADS) a.sum_output[(size_t)t * B + b] = __builtin_nanf("");
+            wait_stores();
+            __syncthreads();
+            if (tid == 0) store_agent(flag, 2);
+            return;
+        }
+    }
+    const bool prob = a.out_mode != I6FBW_OUT_NEG_LOG;
+    const float psign = a.out_mode == I6FBW_OUT_NEG_PROB ? -1.f : 1.f;
+    const int nE = m.n_edges, D = m.D, SP = m.SP, DP = m.DP;
+    const long long soff = state_off(m.edge_begin, b), goff = slot_off(m.edge_begin, b);
+    const uint4* crec = a.crec + m.edge_begin;
+    const int* cb = a.cbegin + goff;
+    const double* offA = a.offA + (size_t)b * T;
+    const double* offB = a.offB + (size_t)b * T;
+    const float* abase = a.alpha + (size_t)T * soff;
+    const float* bbase = a.beta + (size_t)T * soff;
+    const float* gbase = a.gtab + (size_t)T * goff;
+    float* cpbase = fa.cp + (size_t)T * goff;
+
+    // this thread's edges and slots stay in registers for the whole strip
+    constexpr int JE = COMB_FAST_EDGES / COMB_THREADS, JS = COMB_FAST_SLOTS / COMB_THREADS;
+    unsigned eft[JE], esl[JE];
+    float ew[JE];
+#pragma unroll
+    for (int j = 0; j < JE; j++) {
+        const int i = tid + j * COMB_THREADS;
+        uint4 r = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+        if (i < nE) r = crec[i];
+        eft[j] = r.x; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
+    }
+    unsigned cr[JS];          // first edge | one past the last edge << 16 of my slots
+#pragma unroll
+    for (int js = 0; js < JS; js++) {
+        const int d = tid + js * COMB_THREADS;
+        cr[js] = d < D ? (unsigned)cb[d] | ((unsigned)cb[d + 1] << 16) : 0u;
+    }
+    // the operands of the next frame are fetched while the current one is processed
+    float va[JE], vb[JE], vg[JE];
+    double voff = 0.0;
+    auto fetch = [&](int t) {
+        const float* arow = abase + (size_t)t * SP;
+        const float* brow = bbase + (size_t)t * SP;
+        const float* grow = gbase + (size_t)t * DP;
+#pragma unroll
+        for (int j = 0; j < JE; j++) {
+            va[j] = load_x<SYNC>(arow + (eft[j] & 0xFFFFu)); vb[j] = load_x<SYNC>(brow + (eft[j] >> 16)); vg[j] = load_x<SYNC>(grow + esl[j]);
+        }
+        if (tid == 0) voff = load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t);
+    };
+    fetch(t0);
+    for (int t = t0; t < tv; t++) {
+        // edge scores x = alpha_t[from] + w + am + beta_{t+1}[to]   (fbw_op.cu:93-100)
+        float x[JE];
+        float lmin = INF_F;
+#pragma unroll
+        for (int j = 0; j < JE; j++) { x[j] = (va[j] + ew[j]) + (vg[j] + vb[j]); lmin = fminf(lmin, x[j]); }
+        const double offs = voff;
+        if (t + 1 < tv) fetch(t + 1);
+        const float mn = block_min256(lmin, redmin);
+#pragma unroll
+        for (int j = 0; j < JE; j++) xs[tid + j * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
+        __syncthreads();
+        // per-emission sums in fixed (input) order, then the frame normaliser (fbw_op.cu:115-134)
+        float sd[JS];
+        float lsum = 0.f;
+#pragma unroll
+        for (int js = 0; js < JS; js++) {
+            sd[js] = slot_sum(xs, (int)(cr[js] & 0xFFFFu), (int)(cr[js] >> 16));
+            lsum += sd[js];
+        }
+        const float tot = block_sum256(lsum, redsum);
+        const bool dead = mn == INF_F;
+        const float logtot = __builtin_amdgcn_logf(tot);
+        if (tid == 0)
+            a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)(((double)(mn - logtot) + offs) * (double)LN2);
+        const float inv = dead ? 0.f : psign / tot;
+        float* cprow = cpbase + (size_t)t * DP;
+#pragma unroll
+        for (int js = 0; js < JS; js++) {
+            const int d = tid + js * COMB_THREADS;
+            if (d < D) {
+                float v;
+                if (prob) v = sd[js] * inv;
+                else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+                store_agent(cprow + d, v);
+            }
+        }
+    }
+    wait_stores();
+    __syncthreads();
+    if (tid == 0) store_agent(flag, 1);
+}
+
+// Rows [row0, row1) of the tensor in memory order are this group's (frames [t0, ...) of all
+// sequences in layout 0, of sequence bg in layout 1); this job writes the spans job, job + nW,
+// job + 2 nW, ... of the group: jobs that run side by side then write neighbouring spans, i.e. one
+// contiguous window of memory that moves on as they move on (consecutive spans per job -- a window
+// of scattered pieces -- measured slower).  All a job needs from memory is fetched up front in two
+// rounds -- the records of the sequences whose rows its spans cut, their flags and the slot ranges
+// of its pieces of those rows; then emission index and posterior of every slot in those ranges
+// (into registers) -- so that the spans themselves go out back to back: scatter the values that
+// fall into the span into the LDS image, read it back in 16-byte chunks, store, clear.  A span of
+// FLAT_W <= F floats cuts at most two rows.
+template <bool SYNC>
+__device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long row0, const long long row1, const int t0, const int bg,
+                                           const int job, float4a* img4, int* s_row, long long* s_off) {
+    const CombArgs& a = fa.c;
+    const int tid = threadIdx.x;
+    const int T = a.T, B = a.B, F = a.F;
+    const long long g0 = row0 * F + fa.shift, g1 = row1 * F + fa.shift;     // in the line-aligned view (base = out - shift)
+    const long long first = g0 & ~31LL;                                     // first span of the group
+    const int group_spans = (int)((g1 - first + FLAT_W - 1) / FLAT_W);
+    if (job >= group_spans) return;
+    const int nspans = min(FLAT_KMAX, (group_spans - job + fa.nW - 1) / fa.nW);
+#ifdef I6_TRACE
+    const bool traced = (blockIdx.x % 997) == 5 && blockIdx.x / 997 < 60 && tid == 0;
+    unsigned long long* tr = g_trace + 2048 + (blockIdx.x / 997) * 16;
+    if (traced) { tr[0] = wall_clock64(); tr[15] = blockIdx.x; }
+#endif
+    float* image = (float*)img4;
+    const float hole = a.out_mode != I6FBW_OUT_NEG_LOG ? 0.f : INF_F;
+    const float4a hole4 = {hole, hole, hole, hole};
+    static_assert(FLAT_W / 4 == 2 * COMB_THREADS, "two chunks per thread");
+    img4[tid] = hole4;
+    img4[tid + COMB_THREADS] = hole4;
+    // per (span, first or second row it cuts): what the piece is made of (-1 no such piece, 0 holes
+    // only, 1 compact posteriors, 2 NaN, 3 left to fbw_combine), its place in the span, and for kind 1
+    // the slot range of the piece and where the slots' emission indices and values are
+    int* s_kind = s_row;
+    int* s_lo = s_row + 2 * FLAT_KMAX;
+    int* s_hi = s_row + 4 * FLAT_KMAX;
+    int* s_at = s_row + 6 * FLAT_KMAX;      // position of emission 0 of the row relative to the span (may be negative)
+    int* s_p0 = s_row + 8 * FLAT_KMAX;      // piece [s_p0, s_p1) of the span
+    int* s_p1 = s_row + 10 * FLAT_KMAX;
+    long long* s_de = s_off;
+    long long* s_cp = s_off + 2 * FLAT_KMAX;
+    if (tid < 2 * nspans) {
+        const int k = tid >> 1;
+        const long long span0 = first + (long long)(job + k * fa.nW) * FLAT_W;
+        const long long lo = max(span0, g0), hi = min(span0 + FLAT_W, g1);
+        // (a group holds fewer than 2^31 floats: the host sees to that)
+        const unsigned rr = (unsigned)(lo - g0) / (unsigned)F + (tid & 1);          // row within the group
+        const long long rbeg = g0 + (long long)rr * F;
+        const long long pl = max(lo, rbeg), ph = min(hi, rbeg + F);
+        int kind = -1, s0 = 0, s1 = 0;
+        if (pl < ph) {
+            const int t = fa.layout == 0 ? t0 + (int)(rr / (unsigned)B) : t0 + (int)rr;
+            const int b = fa.layout == 0 ? (int)(rr % (unsigned)B) : bg;
+            // everything is requested before the first answer is looked at
+            const SeqMeta m = a.meta[b];
+            const int* wp = fa.wpfx + (size_t)b * fa.wpfx_stride;
+            const int w0 = wp[(int)(pl - rbeg) >> 5], w1 = wp[((int)(ph - rbeg) + 31) >> 5];
+            const int* flag = fa.cflag + (size_t)b * ((T + FLAT_TCF - 1) / FLAT_TCF) + t / FLAT_TCF;
+            const int f0 = load_agent(flag);
+            kind = 0;
+            if (t < m.L) {
+                if (seq_error(m) < 0) kind = 2;
+                else if (m.n_edges == 0) kind = 0;
+                else if (!flat_fast(m)) kind = 3;
+                else {
+                    s0 = w0; s1 = w1;
+                    const long long goff = slot_off(m.edge_begin, b);
+                    s_de[tid] = goff;
+                    s_cp[tid] = (long long)T * goff + (long long)t * m.DP;
+                    kind = (f0 >= 1 || spin_until_ge(flag, 1, a.sync)) && load_agent(flag) == 1 ? 1 : 2;
+                }
+            }
+        }
+        s_kind[tid] = kind; s_lo[tid] = s0; s_hi[tid] = s1;
+        s_at[tid] = (int)(rbeg - span0); s_p0[tid] = (int)(pl - span0); s_p1[tid] = (int)(ph - span0);
+    }
+    __syncthreads();
+#ifdef I6_TRACE
+    if (traced) tr[1] = wall_clock64();
+#endif
+    // Slots of the pieces -> registers.  Piece i belongs to the LP lanes from i * LP on; each of them
+    // takes every LP-th slot of the piece, up to NSP of them: position within the span (-1: none)
+    // and value.  A piece with more slots than that (rare: more than a thirty-second of its emissions
+    // in use) is completed in the span loop below.
+    constexpr int LP = COMB_THREADS / (2 * FLAT_KMAX), NSP = 8;
+    static_assert(LP * 2 * FLAT_KMAX == COMB_THREADS && LP >= 1, "lanes per piece");
+    const int mine = tid / LP, ln = tid % LP;          // my piece, my lane within it
+    int q[NSP];
+    float v[NSP];
+    const bool have = mine < 2 * nspans && s_kind[mine] == 1;
+    {
+        // (all loads are issued before the first result is used: index and value do not depend on each other)
+        const int s0 = have ? s_lo[mine] : 0, s1 = have ? s_hi[mine] : 0;
+        const int* de = a.demis + (have ? s_de[mine] : 0);
+        const float* cprow = fa.cp + (have ? s_cp[mine] : 0);
+#pragma unroll
+        for (int n = 0; n < NSP; n++) {
+            const int sl = s0 + ln + n * LP;
+            q[n] = -1; v[n] = 0.f;
+            if (sl < s1) { q[n] = de[sl]; v[n] = load_agent(cprow + sl); }
+        }
+        const int at = have ? s_at[mine] : 0, p0 = have ? s_p0[mine] : 0, p1 = have ? s_p1[mine] : 0;
+#pragma unroll
+        for (int n = 0; n < NSP; n++) {
+            if (q[n] >= 0) {
+                const int pos = at + q[n];
+                q[n] = (pos >= p0 && pos < p1) ? pos : -1;
+            }
+        }
+    }
+    bool crowded = false;
+    for (int i = 0; i < 2 * nspans; i++) crowded = crowded || (s_kind[i] == 1 && s_hi[i] - s_lo[i] > LP * NSP);
+    float* dst0 = (a.out - fa.shift) + first;
+#ifdef I6_TRACE
+    if (traced) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); tr[2] = wall_clock64(); }
+#endif
+#pragma unroll
+    for (int k = 0; k < FLAT_KMAX; k++) {
+        if (k >= nspans) break;
+        const long long span0 = first + (long long)(job + k * fa.nW) * FLAT_W;
+        const int ka = s_kind[2 * k], kb = s_kind[2 * k + 1];
+        // Spans that need care: cut by an end of the group, or holding a piece that is constant (NaN) or
+        // not written here.  All others -- nearly all -- take the short way: a handful of LDS writes, two
+        // LDS reads, two stores.
+        const bool special = span0 < g0 || span0 + FLAT_W > g1 || ka >= 2 || kb >= 2;
+        if (special) {
+#pragma unroll
+            for (int w = 0; w < 2; w++) {
+                const int kind = w ? kb : ka;
+                if (kind < 2) continue;
+                const float c = kind == 2 ? __builtin_nanf("") : __uint_as_float(FLAT_SKIP);
+                for (int i = s_p0[2 * k + w] + tid; i < s_p1[2 * k + w]; i += COMB_THREADS) image[i] = c;
+            }
+            // elements of the span outside the group belong to the neighbouring group
+            for (int i = tid; i < (int)(g0 - span0); i += COMB_THREADS) image[i] = __uint_as_float(FLAT_SKIP);
+            for (int i = (int)max(0LL, g1 - span0) + tid; i < FLAT_W; i += COMB_THREADS) image[i] = __uint_as_float(FLAT_SKIP);
+        }
+        // the image holds holes everywhere else (see below); now my values of this span
+        if ((mine >> 1) == k) {
+#pragma unroll
+            for (int n = 0; n < NSP; n++)
+                if (q[n] >= 0) image[q[n]] = v[n];
+        }
+        if (crowded) {
+            for (int w = 0; w < 2; w++) {
+                const int i = 2 * k + w;
+                if (s_kind[i] != 1) continue;
+                for (int sl = s_lo[i] + LP * NSP + tid; sl < s_hi[i]; sl += COMB_THREADS) {
+                    const int pos = s_at[i] + a.demis[s_de[i] + sl];
+                    if (pos >= s_p0[i] && pos < s_p1[i]) image[pos] = load_agent(fa.cp + s_cp[i] + sl);
+                }
+            }
+        }
+        lds_barrier();
+        float4a c4[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) c4[u] = img4[tid + u * COMB_THREADS];
+        float* d0 = dst0 + (size_t)(job + k * fa.nW) * FLAT_W + 4 * tid;
+        if (!special) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) I6_ROW_STORE(c4[u], (float4a*)(d0 + 4 * u * COMB_THREADS));
+        } else {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                float* d = d0 + 4 * u * COMB_THREADS;
+                const bool whole = __float_as_uint(c4[u].x) != FLAT_SKIP && __float_as_uint(c4[u].y) != FLAT_SKIP &&
+                                   __float_as_uint(c4[u].z) != FLAT_SKIP && __float_as_uint(c4[u].w) != FLAT_SKIP;
+                if (whole) I6_ROW_STORE(c4[u], (float4a*)d);
+                else {
+                    if (__float_as_uint(c4[u].x) != FLAT_SKIP) d[0] = c4[u].x;
+                    if (__float_as_uint(c4[u].y) != FLAT_SKIP) d[1] = c4[u].y;
+                    if (__float_as_uint(c4[u].z) != FLAT_SKIP) d[2] = c4[u].z;
+                    if (__float_as_uint(c4[u].w) != FLAT_SKIP) d[3] = c4[u].w;
+                }
+            }
+        }
+        // every thread clears the chunks it has read: holes everywhere again
+        img4[tid] = hole4;
+        img4[tid + COMB_THREADS] = hole4;
+        lds_barrier();
+#ifdef I6_TRACE
+        if (traced) tr[3 + k] = wall_clock64();
+#endif
+    }
+#ifdef I6_TRACE
+    if (traced) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); tr[12] = wall_clock64(); }
+#endif
+}
+
+template <bool SYNC>
+__global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs fa) {
+    __shared__ float4a img4[FLAT_W / 4];        // image of a write job; staging area of a posterior job
+    __shared__ float redmin[COMB_THREADS / 64];
+    __shared__ float redsum[COMB_THREADS / 64];
+    __shared__ int s_kind[12 * FLAT_KMAX];
+    __shared__ long long s_off[4 * FLAT_KMAX];
+    static_assert(FLAT_W >= COMB_FAST_EDGES, "the staging area of a posterior job lies in the image");
+    const int B = fa.c.B, T = fa.c.T;
+    const int n = (T + TC - 1) / TC;
+    // job of this workgroup
+    constexpr int NQ = TC / FLAT_TCF;           // posterior jobs per strip of a sequence
+    int i, b = -1, job = -1, qf = 0;            // job >= 0: write job number within its group; qf: which part of the strip
+    const int blk = blockIdx.x;
+    if (blk < FLAT_AHEAD * B * NQ) { i = blk / (B * NQ); b = (blk / NQ) % B; qf = blk % NQ; }
+    else {
+        const int x = blk - FLAT_AHEAD * B * NQ;
+        const int G = fa.nW + (fa.layout == 0 ? B : 1) * NQ;
+        const int u = x / G, r = x % G;
+        if (fa.layout == 0) { i = u; if (r < fa.nW) job = r; else { b = (r - fa.nW) / NQ; qf = (r - fa.nW) % NQ; i += FLAT_AHEAD; } }
+        else { i = u / B; b = u % B; if (r < fa.nW) job = r; else { qf = r - fa.nW; i += FLAT_AHEAD; } }
+    }
+#ifdef I6_TRACE
+    if (blk == 0 && threadIdx.x == 0) g_trace[2040] = wall_clock64();
+#endif
+    if (i >= n) return;
+    // middle: where the two recursions meet -- of the longest sequence (rows of all sequences of a
+    // frame lie side by side) or of this sequence
+    const int Lmid = fa.layout == 0 ? fa.c.sync[6] : fa.c.meta[b].L;
+    const int strip = middle_out(i, n, min(n - 1, (Lmid / 2) / TC));
+    if (job < 0) {
+        flat_post<SYNC>(fa, b, strip * TC + qf * FLAT_TCF, (float*)img4, redmin, redsum, s_kind);
+        return;
+    }
+    const long long row0 = fa.layout == 0 ? (long long)strip * TC * B : (long long)b * T + strip * TC;
+    const long long row1 = fa.layout == 0 ? (long long)min(T, strip * TC + TC) * B : (long long)b * T + min(T, strip * TC + TC);
+    flat_write<SYNC>(fa, row0, row1, strip * TC, b, job, img4, s_kind, s_off);
+}
+
 // Status of a call in two ints {code, sequence}: the first sequence with a reported problem, else a
 // timeout of the hand-off between kernels, else ok.  One workgroup.
 __global__ __launch_bounds__(256) void fbw_status_reduce(const SeqMeta* meta, int B, const int* sync, int* out2) {
@@ -1873,6 +2341,7 @@ int device_init(Pipeline& p) {
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     hipFuncAttributes attr;
+    HIP_TRY(hipFuncSetAttribute((const void*)fbw_flat<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 0));
     HIP_TRY(hipFuncGetAttributes(&attr, (const void*)fbw_recurse_dense<true>));
     p.dense_regs = attr.numRegs;
     // address of the current device's copy of the built-in workspace
@@ -1947,6 +2416,7 @@ struct StageTimer {
     }
 };
 
+int row_misalign_host(const float* p) { return (int)(((uintptr_t)p >> 2) & 31); }
 size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_XS * 4; }
 constexpr int COMB_TILE_W = 12288;     // floats of a row that go through LDS at a time when the row does not fit: three workgroups per unit
 
@@ -1955,6 +2425,13 @@ std::atomic<int> g_no_band{0};      // see i6fbw_set_band
 std::atomic<int> g_overlap_mode{[] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
+}()};
+
+// dense writer: -1 by problem (flat spans where the layout allows it and the stages overlap), 0 always row by row,
+// 1 flat wherever the layout allows it; I6FBW_DENSE_WRITER=rows|flat sets the initial value
+std::atomic<int> g_writer_mode{[] {
+    const char* e = getenv("I6FBW_DENSE_WRITER");
+    return e ? (e[0] == 'r' ? 0 : 1) : -1;
 }()};
 
 // Status reports that travel to the host without a wait: per device a ring of pinned {code, seq}
@@ -2002,7 +2479,7 @@ extern "C" {
 
 int i6fbw_workspace_size(int T, int B, int F, int E, int n_states, size_t* bytes) {
     if (!bytes || T <= 0 || B <= 0 || F <= 0 || E < 0 || n_states <= 0) return I6FBW_ERR_INVALID_ARGUMENT;
-    *bytes = make_layout(T, B, E).total;
+    *bytes = make_layout(T, B, E, F).total;
     return I6FBW_OK;
 }
 
@@ -2063,7 +2540,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     if (out_stride_t < 0 || out_stride_b < 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
-    const Layout l = make_layout(T, B, E);
+    const Layout l = make_layout(T, B, E, F);
     if (static_call) {
         if (l.total > (size_t)I6FBW_STATIC_WORKSPACE_BYTES) return I6FBW_ERR_STATIC_WORKSPACE;
     } else if (workspace_bytes < l.total) return I6FBW_ERR_WORKSPACE_TOO_SMALL;
@@ -2125,6 +2602,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx); pa.renum = (int2*)(ws + l.renum);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
+    pa.cflag = (int*)(ws + l.cflag); pa.wpfx = l.wpfx_stride > 0 ? (int*)(ws + l.wpfx) : nullptr; pa.wpfx_stride = l.wpfx_stride;
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
@@ -2144,10 +2622,34 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     ca.alpha = ra.alpha; ca.beta = ra.beta; ca.gtab = ga.gtab; ca.offA = ra.offA; ca.offB = ra.offB;
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     ca.tile_w = tiled ? COMB_TILE_W : 0;
+    ca.direct_only = 0;
     // More recursion workgroups than compute units: the instance of which two fit on a unit -- unless
     // the sequences can be longer than 4096 frames, which only the other instance runs in double
     // precision (recurse_workgroup); it then takes two rounds.
     const bool dense = 2 * B > P.n_cu && T <= 4096;
+    // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
+    // order of frames and sequences, rows are long enough for a span to cut only a few of them,
+    // and the stages overlap (for the small problems of the single-stream schedule the row writer
+    // is as good).
+    int flat_layout = -1;
+    if (out_stride_b == (int64_t)F && out_stride_t == (int64_t)B * F) flat_layout = 0;
+    else if (out_stride_t == (int64_t)F && out_stride_b == (int64_t)T * F) flat_layout = 1;
+    const int writer = g_writer_mode.load();
+    bool flat = (writer > 0 || (writer < 0 && overlap)) && flat_layout >= 0 && F >= FLAT_MIN_F && l.wpfx_stride > 0;
+    FlatArgs fa;
+    long long flat_grid = 0;
+    if (flat) {
+        const long long n = (T + TC - 1) / TC, rows = flat_layout == 0 ? B : 1;
+        fa.c = ca; fa.layout = flat_layout;
+        fa.K = FLAT_KMAX;
+        fa.nW = (int)(((long long)TC * rows * F + 31 + (long long)fa.K * FLAT_W - 1) / ((long long)fa.K * FLAT_W));
+        fa.shift = row_misalign_host(out);
+        fa.cflag = (int*)(ws + l.cflag); fa.wpfx = (const int*)(ws + l.wpfx); fa.wpfx_stride = l.wpfx_stride;
+        fa.cp = ga.gtab;
+        flat_grid = (long long)FLAT_AHEAD * B * (TC / FLAT_TCF) + (flat_layout == 0 ? n : n * B) * (fa.nW + rows * (TC / FLAT_TCF));
+        if (flat_grid > 0x7fffffffLL || (long long)TC * rows * F >= (1LL << 31) - FLAT_W) flat = false;
+    }
+    ca.direct_only = flat ? 1 : 0;
 
     {
         // the scan also clears the header of the hand-off area, so it runs even without edges
@@ -2191,9 +2693,20 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
         HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
         int rc = launch_recursion(); if (rc != I6FBW_OK) return rc;
     }
-    // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
-    // leaves the memory system idle.
-    {
+    if (flat && overlap) {
+        // fbw_flat writes every row except those of sequences too large for its posterior jobs:
+        // these go row by row through fbw_combine on the second library stream, started once the
+        // preparation is done and all recursion workgroups are placed (its workgroups wait for the
+        // gather and the recursion while they hold wave slots); it has nothing to do for the usual
+        // batch.  The two kernels do not wait for each other.
+        if (early) HIP_TRY(hipEventRecord(P.fork, s));
+        HIP_TRY(hipStreamWaitEvent(sP, P.fork, 0));
+        hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sP, sync, 2 * B);
+        { StageTimer tm(4, sP, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, sP, ca); }
+        HIP_TRY(hipGetLastError());
+    } else if (!flat) {
+        // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
+        // leaves the memory system idle.
         StageTimer tm(4, sP, timed);
         hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
                            (long long)out_stride_b, sum_output);
@@ -2207,7 +2720,11 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
         { StageTimer tm(2, s, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, s, ra);
           else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
-        { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+        if (flat) {
+            // (the row kernel first: it only has the sequences that are too large for the other one)
+            { StageTimer tm(4, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+            { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_flat<false>, dim3((unsigned)flat_grid), dim3(COMB_THREADS), 0, s, fa); }
+        } else { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
         HIP_TRY(hipGetLastError());
         return I6FBW_OK;
     }
@@ -2226,7 +2743,8 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
 #ifdef I6_TRACE
     if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
 #endif
-    { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+    if (flat) { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_flat<true>, dim3((unsigned)flat_grid), dim3(COMB_THREADS), 0, s, fa); }
+    else { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
     HIP_TRY(hipGetLastError());
     // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
@@ -2337,6 +2855,8 @@ const char* i6fbw_strerror(int code) {
         default: return "unknown status";
     }
 }
+
+void i6fbw_set_dense_writer(int mode) { g_writer_mode = mode < 0 ? -1 : (mode ? 1 : 0); }
 
 void i6fbw_set_overlap(int mode) {
     std::lock_guard<std::mutex> lock(g_mutex);

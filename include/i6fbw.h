@@ -219,6 +219,17 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
 void i6fbw_set_overlap(int mode);
 
 /*
+ * Chooses how i6fbw_run writes the dense (T, B, F) tensor: 0 row by row (one workgroup per strip of
+ * frames of a sequence builds each row in LDS and streams it out), 1 in flat 128-byte-aligned spans
+ * fed from compact per-frame posteriors wherever the output is one contiguous block ((T, B, F) or
+ * (B, T, F) order, F >= 128), -1 (default) flat spans for the large problems whose stages overlap.
+ * The environment variable I6FBW_DENSE_WRITER=rows|flat sets the initial value.  Results do not
+ * depend on the writer.  No counterpart in the reference (fbw_op.cu:137-153,366-377 scatter with
+ * atomics into a pre-filled tensor).
+ */
+void i6fbw_set_dense_writer(int mode);
+
+/*
  * Device-side construction of the automaton arrays for two common topologies.  No counterpart in
  * the reference, which leaves the tuple (number of states, edges, weights, start/end states) to
  * its callers (fbw/__init__.py:56-62); these take that step off the host.  States of sequence b
