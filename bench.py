@@ -8,10 +8,13 @@ recursion, per-frame normalisation and the dense (T,B,F) posterior write.
 
 Prints ONE JSON line.  `value` is the achieved algorithmic bandwidth of the whole call
 (bytes = 4*T*B*F + 4*sum_b seq_len_b*E_b + 20*E + 4*T*B + 12*B, every datum once);
-`ms_per_step` is ms per loss+grad call.  `roofline` prices the dominant kernel (the combine
-kernel that writes the dense tensor) against 8 TB/s with durations taken from HIP events on
-the stream it runs on; `cpu_baseline` times the fp32 CPU port of the reference algorithm
-(oracle/fbw_oracle.c) on the host cores in the same run.
+`ms_per_step` is ms per loss+grad call.  `roofline` prices the dominant kernel (the one that
+writes the dense tensor: fbw_flat, or fbw_combine where the row writer runs) against 8 TB/s with
+durations taken from HIP events on the stream it runs on; `cpu_baseline` times the fp32 CPU port
+of the reference algorithm (oracle/fbw_oracle.c) on the host cores in the same run, with all
+cores and with one; `config.per_config` holds, for each of the five benchmark configurations,
+the time per call (median and minimum over single calls timed with HIP events), the roofline
+fraction, sequence-frames per second and the worst loss / posterior error against the fp64 oracle.
 """
 import argparse
 import json
@@ -23,6 +26,92 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+NAMES = ["tiny", "monophone", "cart", "ctc", "longform"]
+
+
+class Problem:
+    """One workload resident on the device, called through the C ABI."""
+
+    def __init__(self, W, out_mode):
+        import torch
+        from i6_native_ops_amd import cabi
+        self.W, self.out_mode, self.cabi, self.torch = W, out_mode, cabi, torch
+        dev = torch.device("cuda:0")
+        self.am = torch.from_numpy(W.am_scores).to(dev)
+        self.edges = torch.from_numpy(W.edges).to(dev)
+        self.weights = torch.from_numpy(W.weights).to(dev)
+        self.start_end = torch.from_numpy(W.start_end_states).to(dev)
+        self.seq_lens = torch.from_numpy(W.seq_lens).to(dev)
+        self.out = torch.empty((W.T, W.B, W.F), dtype=torch.float32, device=dev)
+        self.loss = torch.empty((W.T, W.B), dtype=torch.float32, device=dev)
+        self.ws_bytes = cabi.workspace_size(W.T, W.B, W.F, W.E, W.n_states)
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def step(self):
+        W = self.W
+        self.cabi.run(self.am.data_ptr(), self.am.stride(0), self.am.stride(1), self.edges.data_ptr(), self.edges.stride(0),
+                      self.weights.data_ptr(), self.start_end.data_ptr(), self.start_end.stride(0), self.seq_lens.data_ptr(),
+                      W.T, W.B, W.F, W.E, W.n_states, self.out_mode, self.out.data_ptr(), self.loss.data_ptr(),
+                      self.ws.data_ptr(), self.ws_bytes, self.stream)
+
+    def check(self):
+        code, seq = self.cabi.read_status(self.ws.data_ptr(), self.W.B, self.stream)
+        if code != 0:
+            raise self.cabi.FbwError(code, seq)
+
+    def single_call_times(self, n, warmup):
+        """ms of n single calls, each bracketed by HIP events on the stream the call is made on (the
+        library joins its own streams into it before the call returns)"""
+        torch = self.torch
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, b in ev:
+            a.record()
+            self.step()
+            b.record()
+        torch.cuda.synchronize()
+        return sorted(a.elapsed_time(b) for a, b in ev)
+
+
+def cpu_threads(W, fbw_oracle):
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    return max(1, min(W.B, cores, fbw_oracle.max_threads()))
+
+
+def per_config_entry(name, headline=None):
+    """Timing and parity of one benchmark configuration (the headline's device problem is reused)."""
+    import numpy as np
+    from i6_native_ops_amd.fbw.workloads import make_workload
+    from oracle import fbw_oracle
+    P = headline if headline is not None else Problem(make_workload(name), 1)
+    W = P.W
+    P.step()
+    P.check()
+    times = P.single_call_times(30, 5)
+    med, mn = times[len(times) // 2], times[0]
+    alg = W.algorithmic_bytes()
+    # parity against the fp64 oracle at full size: relative error of the loss, absolute error of the posteriors
+    want_out, want_loss = fbw_oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states,
+                                                threads=cpu_threads(W, fbw_oracle))
+    loss = P.loss.cpu().numpy()
+    nz = want_loss != 0
+    loss_err = float(np.max(np.abs(loss[nz] - want_loss[nz]) / np.abs(want_loss[nz]))) if nz.any() else 0.0
+    post_err = 0.0
+    out = P.out.cpu().numpy()
+    for t0 in range(0, W.T, 64):          # in slices: exp of the whole oracle tensor at once doubles the host memory
+        post_err = max(post_err, float(np.max(np.abs(out[t0:t0 + 64] - np.exp(-want_out[t0:t0 + 64].astype(np.float64))))))
+    return {"T": W.T, "B": W.B, "F": W.F, "E": W.E, "ms_median": round(med, 4), "ms_min": round(mn, 4),
+            "algorithmic_bytes": alg, "gbps": round(alg / (med * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(alg / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "seq_frames_per_s": round(W.seq_frames() / (med * 1e-3), 1),
+            "loss_rel_err": float("%.3g" % loss_err), "posterior_abs_err": float("%.3g" % post_err)}
 
 
 def main():
@@ -34,6 +123,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-wrapper", action="store_true", help="skip the wrapper-level (fbw_loss + backward) timing")
     ap.add_argument("--no-best-path", action="store_true", help="skip the best-path (Viterbi) timing")
+    ap.add_argument("--no-per-config", action="store_true",
+                    help="skip the per-configuration table (timings and errors against the oracle for all five workloads)")
     ap.add_argument("--out-mode", type=int, default=1, help="0: -log posterior with +inf holes, 1: posterior")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise copy kernel over 1 GiB (3 times) so that a rocprofv3 --pmc run of "
@@ -55,22 +146,11 @@ def main():
     cabi.load()   # fails loudly if the HIP library is not built
 
     W = make_workload(args.workload)
+    P = Problem(W, args.out_mode)
     dev = torch.device("cuda:0")
-    am = torch.from_numpy(W.am_scores).to(dev)
-    edges = torch.from_numpy(W.edges).to(dev)
-    weights = torch.from_numpy(W.weights).to(dev)
-    start_end = torch.from_numpy(W.start_end_states).to(dev)
-    seq_lens = torch.from_numpy(W.seq_lens).to(dev)
-    out = torch.empty((W.T, W.B, W.F), dtype=torch.float32, device=dev)
-    loss = torch.empty((W.T, W.B), dtype=torch.float32, device=dev)
-    ws_bytes = cabi.workspace_size(W.T, W.B, W.F, W.E, W.n_states)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def step():
-        cabi.run(am.data_ptr(), am.stride(0), am.stride(1), edges.data_ptr(), edges.stride(0), weights.data_ptr(),
-                 start_end.data_ptr(), start_end.stride(0), seq_lens.data_ptr(), W.T, W.B, W.F, W.E, W.n_states,
-                 args.out_mode, out.data_ptr(), loss.data_ptr(), ws.data_ptr(), ws_bytes, stream)
+    am, edges, weights, start_end, seq_lens, ws, ws_bytes, stream = (P.am, P.edges, P.weights, P.start_end, P.seq_lens, P.ws,
+                                                                      P.ws_bytes, P.stream)
+    step = P.step
 
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).fill_(1.0)
@@ -81,9 +161,7 @@ def main():
         del src, dst
 
     step()
-    code, seq = cabi.read_status(ws.data_ptr(), W.B, stream)
-    if code != 0:
-        raise cabi.FbwError(code, seq)
+    P.check()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -103,25 +181,28 @@ def main():
     torch.cuda.synchronize()
     _, stage_ms = cabi.profile_read()
     cabi.profile_enable(False)
+    flat = cabi.last_dense_writer() == 1
 
     alg_bytes = W.algorithmic_bytes()
     gbps = alg_bytes / (ms_per_call * 1e-3) / 1e9
-    # dominant kernel: fbw_combine, which writes the F-wide posterior row and the loss of every frame
-    # that carries probability mass: (4*F + 4) bytes per row, sum_b seq_len_b rows per call, spread
-    # over the combine launches of one call (their durations are summed; fbw_padfill writes the
-    # remaining rows and is timed separately)
-    comb_bytes = (4 * W.F + 4) * W.seq_frames()
+    # Dominant kernel: the one that writes the dense tensor.  fbw_flat writes all T*B rows of F floats and
+    # the loss of every frame, 4*T*B*F + 4*T*B bytes per launch; where the row writer runs, fbw_combine
+    # writes the rows of the frames that carry probability mass, (4*F + 4) bytes each, sum_b seq_len_b
+    # rows per launch (fbw_padfill writes the others and is timed separately).
+    kernel = "fbw_flat" if flat else "fbw_combine"
+    comb_bytes = 4 * W.T * W.B * W.F + 4 * W.T * W.B if flat else (4 * W.F + 4) * W.seq_frames()
     comb_ms = stage_ms[3]
     comb_gbps = comb_bytes / (comb_ms * 1e-3) / 1e9 if comb_ms > 0 else 0.0
-    # HBM bytes per call of the dominant kernel, from the committed rocprofv3 --pmc summary
-    # (FETCH_SIZE and WRITE_SIZE, each scaled by what it reads for a copy kernel of known size)
-    traffic = None
+    # HBM bytes per launch of that kernel: not measured in this run (counters need the profiler); the
+    # figure comes from the committed rocprofv3 --pmc summary of this command and names it
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", f"fbw_{args.workload}_hbm_traffic.txt")
     if os.path.exists(tpath):
         import re
-        m = re.search(r"fbw_combine, scaled:.*= ([0-9.]+) MB per launch", open(tpath).read())
+        m = re.search(kernel + r", scaled:.*= ([0-9.]+) MB per launch", open(tpath).read())
         if m:
             traffic = int(float(m.group(1)) * 1e6)
+            traffic_source = f"profiles/fbw_{args.workload}_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, committed)"
 
     result = {
         "metric": f"FBW loss+grad ms/call + achieved HBM GB/s at T={W.T},B={W.B},F={W.F} fp32",
@@ -137,15 +218,16 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: T={W.T} B={W.B} F={W.F} E={W.E} states={W.n_states}, "
-                               f"seed={1001 + ['tiny', 'monophone', 'cart', 'ctc', 'longform'].index(args.workload)}",
+                               f"seed={1001 + NAMES.index(args.workload)}",
                    "out_mode": "posterior" if args.out_mode == 1 else "neg_log",
                    "algorithmic_bytes": alg_bytes,
                    "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
                    "seq_frames_per_s": round(W.seq_frames() / (ms_per_call * 1e-3), 1),
                    "stage_ms": {k: round(v, 4) for k, v in zip(cabi.STAGE_NAMES, stage_ms)}},
-        "roofline": {"bound": "hbm", "kernel": "fbw_combine", "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "algorithmic_bytes_per_call": comb_bytes, "kernel_ms_per_call": round(comb_ms, 4)},
+                     "traffic_source": traffic_source,
+                     "algorithmic_bytes_per_launch": comb_bytes, "kernel_ms_per_launch": round(comb_ms, 4)},
     }
 
     # wrapper level (informational): fbw_loss(log_probs[B,T,F]).sum().backward() with the fused front end
@@ -200,26 +282,39 @@ def main():
 
     if not args.no_cpu_baseline:
         from oracle import fbw_oracle
-        cores = os.cpu_count() or 1
-        try:
-            cores = len(os.sched_getaffinity(0))
-        except AttributeError:
-            pass
-        threads = max(1, min(W.B, cores, fbw_oracle.max_threads()))
-        reps, t_cpu = 0, 0.0
-        while reps < 3 or (t_cpu < 10.0 and reps < 20):
-            t0 = time.perf_counter()
-            fbw_oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states,
-                                  precision="f32", threads=threads)
-            t_cpu += time.perf_counter() - t0
-            reps += 1
-        cpu_ms = t_cpu / reps * 1e3
+        threads = cpu_threads(W, fbw_oracle)
+
+        def cpu_ms(nthreads, budget_s):
+            reps, t_cpu = 0, 0.0
+            while reps < 3 or (t_cpu < budget_s and reps < 20):
+                t0 = time.perf_counter()
+                fbw_oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states,
+                                      precision="f32", threads=nthreads)
+                t_cpu += time.perf_counter() - t0
+                reps += 1
+            return t_cpu / reps * 1e3, reps
+        ms_all, reps = cpu_ms(threads, 10.0)
+        ms_one, reps_one = cpu_ms(1, 0.0)
         result["cpu_baseline"] = {
-            "value": round(alg_bytes / (cpu_ms * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "ms_per_call": round(cpu_ms, 2),
+            "value": round(alg_bytes / (ms_all * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "ms_per_call": round(ms_all, 2),
+            "one_thread": {"value": round(alg_bytes / (ms_one * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": 1,
+                           "ms_per_call": round(ms_one, 2), "calls": reps_one},
             "sample": f"whole {args.workload} workload, {reps} calls of the fp32 CPU port of the reference algorithm "
                       f"(per-frame edge sweeps, normalise, scatter), OpenMP over sequences",
         }
+
+    # all five configurations: time per call and parity against the fp64 oracle at full size
+    if not args.no_per_config:
+        per = {}
+        for name in NAMES:
+            reuse = P if (name == args.workload and args.out_mode == 1) else None
+            if reuse is None and name == args.workload:
+                continue
+            per[name] = per_config_entry(name, reuse)
+            if reuse is None:
+                torch.cuda.empty_cache()
+        result["config"]["per_config"] = per
     print(json.dumps(result))
 
 

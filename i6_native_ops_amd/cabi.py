@@ -13,16 +13,18 @@ LIB_PATH = os.path.join(_HERE, "fbw", "libi6fbw.so")
 OUT_NEG_LOG = 0
 OUT_PROB = 1
 OUT_NEG_PROB = 2
+IN_LOG_PROBS = 1      # am_scores holds log p instead of -log p
+IN_ALL_FRAMES = 2     # gather every (frame, emission) score (needed before an alignment dump)
 N_STAGES = 5
 STAGE_NAMES = ("prepare", "gather", "recurse", "combine", "padfill")
 
 # every symbol include/i6fbw.h declares
 SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read_status", "i6fbw_strerror", "i6fbw_last_hip_error",
-           "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment", "i6fbw_set_band",
+           "i6fbw_set_overlap", "i6fbw_viterbi", "i6fbw_dump_output", "i6fbw_dump_alignment",
            "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
            "i6fbw_profile_enable", "i6fbw_profile_read",
            "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode",
-           "i6fbw_run_static", "i6fbw_static_workspace", "i6fbw_set_dense_writer")
+           "i6fbw_run_static", "i6fbw_static_workspace", "i6fbw_set_dense_writer", "i6fbw_last_dense_writer", "i6fbw_set_spin_limit")
 STATIC_WORKSPACE_BYTES = 32 << 20
 ERR_STATIC_WORKSPACE = -16
 
@@ -63,8 +65,6 @@ def load():
         lib.i6fbw_dump_alignment.argtypes = [c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_void_p, c.c_int64, c.c_float,
                                              c.c_uint, c.c_char_p, c.c_void_p]
         lib.i6fbw_dump_alignment.restype = c.c_int
-        lib.i6fbw_set_band.argtypes = [c.c_int]
-        lib.i6fbw_set_band.restype = None
         lib.i6fbw_ctc_fsa_bounds.argtypes = [c.c_int, c.c_int, c.POINTER(c.c_int), c.POINTER(c.c_int), c.POINTER(c.c_size_t)]
         lib.i6fbw_ctc_fsa_bounds.restype = c.c_int
         lib.i6fbw_build_ctc_fsa.argtypes = [c.c_void_p, c.c_int64, c.c_void_p, c.c_int, c.c_int, c.c_int, c.c_void_p, c.c_int64,
@@ -91,6 +91,10 @@ def load():
         lib.i6fbw_set_overlap.restype = None
         lib.i6fbw_set_dense_writer.argtypes = [c.c_int]
         lib.i6fbw_set_dense_writer.restype = None
+        lib.i6fbw_set_spin_limit.argtypes = [c.c_int]
+        lib.i6fbw_set_spin_limit.restype = c.c_int
+        lib.i6fbw_last_dense_writer.argtypes = []
+        lib.i6fbw_last_dense_writer.restype = c.c_int
         lib.i6fbw_profile_enable.argtypes = [c.c_int]
         lib.i6fbw_profile_enable.restype = None
         lib.i6fbw_profile_read.argtypes = [c.POINTER(c.c_float)]
@@ -142,10 +146,10 @@ def static_workspace():
     return int(ptr.value), int(n.value)
 
 
-def run_strided(am_ptr, am_stride_t, am_stride_b, scores_are_log_probs, edges_ptr, edge_row_stride, weights_ptr,
+def run_strided(am_ptr, am_stride_t, am_stride_b, input_flags, edges_ptr, edge_row_stride, weights_ptr,
                 start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E, n_states, out_mode, out_ptr, out_stride_t,
                 out_stride_b, sum_ptr, ws_ptr, ws_bytes, stream=0) -> None:
-    rc = load().i6fbw_run_strided(am_ptr, am_stride_t, am_stride_b, int(scores_are_log_probs), edges_ptr,
+    rc = load().i6fbw_run_strided(am_ptr, am_stride_t, am_stride_b, int(input_flags), edges_ptr,
                                   edge_row_stride, weights_ptr, start_end_ptr, se_row_stride, seq_lens_ptr, T, B, F, E,
                                   n_states, out_mode, out_ptr, out_stride_t, out_stride_b, sum_ptr, ws_ptr, ws_bytes,
                                   stream)
@@ -197,6 +201,18 @@ def set_dense_writer(mode: int) -> None:
     load().i6fbw_set_dense_writer(int(mode))
 
 
+def set_spin_limit(polls: int) -> None:
+    """Polls before a kernel gives up waiting for another kernel of its call (<= 0: the default)."""
+    rc = load().i6fbw_set_spin_limit(int(polls))
+    if rc != 0:
+        raise FbwError(rc)
+
+
+def last_dense_writer() -> int:
+    """0: the last call wrote the tensor row by row, 1: in flat spans."""
+    return int(load().i6fbw_last_dense_writer())
+
+
 def ctc_fsa_bounds(B, Lmax):
     """(edge capacity, state bound, scratch bytes) that always suffice for i6fbw_build_ctc_fsa."""
     e, n, sb = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_size_t(0)
@@ -223,11 +239,6 @@ def build_hmm_fsa(labels_ptr, label_row_stride, label_lens_ptr, B, Lmax, states_
                                     edge_capacity, weights_ptr, start_end_ptr, se_row_stride, totals_ptr, stream)
     if rc != 0:
         raise FbwError(rc)
-
-
-def set_band(on: bool) -> None:
-    """False: gather every (frame, emission) score, needed before an alignment dump."""
-    load().i6fbw_set_band(1 if on else 0)
 
 
 def dump_alignment(ws_ptr, T, B, E, start_end_ptr, se_row_stride, pruning, batch_idx, directory, stream=0) -> None:

@@ -48,6 +48,9 @@ constexpr int EB_MAX = 8192;          // edges of one sequence (capacity of the 
 constexpr int F_BITMAP_MAX = 131072;  // emission ids covered by the LDS presence bitmap
 constexpr int S_MAX = 4096;           // states of one sequence
 constexpr int D_MAX = 4096;           // distinct emissions of one sequence
+// states of a sequence whose two state vectors fit, as doubles, the state area of the recursion
+// instance that keeps float vectors of S_MAX states (fbw_recurse_dense)
+constexpr int DENSE_F64_STATES = (((S_MAX + 16) / 2 - 16) / 16) * 16;
 #ifndef I6_TG
 #define I6_TG 8
 #endif
@@ -67,6 +70,9 @@ constexpr int COMB_JD = D_MAX / COMB_THREADS;
 constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of the combine kernel
 constexpr int COMB_MID_EDGES = 4096;  // up to here a combine workgroup keeps the edges of its sequence in registers ...
 constexpr int COMB_MID_SLOTS = 2048;  // ... and the distinct emissions of the sequence spread over its threads' registers
+#ifndef I6_FLOAT_FRAMES
+#define I6_FLOAT_FRAMES 512           // sequences with more frames keep their state vectors in double
+#endif
 constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup
 constexpr int REC_LOADERS = 1;        // loader waves beside them
 constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
@@ -82,7 +88,7 @@ constexpr int SYNC_HDR = 16;          // ints before the progress counters in th
                                       // [0] abort flag, [1] recursion workgroups placed so far, [3] preparation workgroups finished,
                                       // [4..5] status report {code, sequence}, [6] longest sequence of the batch in frames
 constexpr int PUBLISH = 32;           // recursion steps between progress publications
-constexpr int SPIN_LIMIT = 1 << 20;   // polls before a waiting wave gives up
+constexpr int SPIN_LIMIT = 1 << 20;   // polls before a waiting wave gives up (see g_spin_limit)
 // Scores are kept in units of log 2 inside the workspace (exp2/log2 are single instructions).
 constexpr float LOG2E = 1.44269504088896341f;
 constexpr float LN2 = 0.693147180559945309f;
@@ -108,8 +114,10 @@ __host__ __device__ inline long long round16(long long x) { return (x + 15) & ~1
 __host__ __device__ inline long long state_off(long long edge_begin, int b) { return round16(2 * edge_begin) + 32LL * b; }
 __host__ __device__ inline long long slot_off(long long edge_begin, int b) { return round16(edge_begin) + 32LL * b; }
 // Entries of a sequence's renumbering table (see local_state) and the home position of a state id in it
-__device__ __forceinline__ unsigned renum_capacity(int n_edges) { return 2u * (2u * (unsigned)n_edges + 16u); }
-__device__ __forceinline__ unsigned renum_home(int id, unsigned cap) { return __umulhi((unsigned)id * 2654435761u, cap); }
+__host__ __device__ inline unsigned renum_capacity(int n_edges) { return 2u * (2u * (unsigned)n_edges + 16u); }
+__host__ __device__ inline unsigned renum_home(int id, unsigned cap) {
+    return (unsigned)(((unsigned long long)((unsigned)id * 2654435761u) * cap) >> 32);
+}
 
 struct Layout {
     size_t meta, sync, sortflag, seqbegin, eidx, ellA, ellB, crec, cbegin, demis, tband, renum, cflag, wpfx, offA, offB, alpha, beta, gtab, total;
@@ -195,10 +203,15 @@ template <bool SYNC, typename T> __device__ __forceinline__ T load_x(const T* p)
 // waits until this wave's global stores have been acknowledged
 __device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// The poll limit is a device variable so that a test can force the give-up path from the host
+// (i6fbw_set_spin_limit) with every kernel still running to its normal end.
+__device__ int g_spin_limit = SPIN_LIMIT;
+
 // polls *p until it is >= want; false if it gave up (or somebody else already had to)
 // (quiet: running out of polls is not an error yet, the caller tries again)
 __device__ __forceinline__ bool spin_until_ge(const int* p, int want, int* abort_flag, bool quiet = false) {
-    for (int n = 0; n < SPIN_LIMIT; n++) {
+    const int limit = g_spin_limit;
+    for (int n = 0; n < limit; n++) {
         if (load_agent(p) >= want) return true;
         if ((n & 255) == 255 && load_agent(abort_flag)) return false;
         __builtin_amdgcn_s_sleep(2);
@@ -257,6 +270,7 @@ struct PrepArgs {
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
     int force_generic;  // F is too large for the emission bitmap: every sequence takes the general path
+    int dense;          // the recursion runs on the instance with the small state area (fbw_recurse_dense)
     int2* renum;        // renumbering tables, two entries per state of room (see local_state)
     SeqMeta* meta; int* sync; int* sortflag; int* seqbegin; int* eidx; uint2* ellA; uint2* ellB; uint4* crec; int* cbegin; int* demis; int2* tband;
     int* cflag = nullptr;   // per (sequence, strip of TC frames): compact posteriors written (flat dense write); may be null
@@ -446,6 +460,10 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     if (n_edges == 0) S = 1;
     if (!err && !sparse && S > S_MAX) generic = 1;
     if (!err && a.force_generic && n_edges > 0) generic = 1;
+    // The recursion instance for batches of more sequences than half the compute units has room for
+    // double-precision state vectors of DENSE_F64_STATES states only: a larger sequence that needs them
+    // (recurse_workgroup) takes the general path, which keeps its vectors in double in memory.
+    if (!err && a.dense && !a.best_path && S > DENSE_F64_STATES && (5LL * S > 3LL * L || L > I6_FLOAT_FRAMES)) generic = 1;
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
     // i-th edge of this sequence in input order
@@ -876,6 +894,7 @@ struct RecCursor {
     double* op; int ostep;           // its offset
     double c; bool pending;          // running offset, renormalisation requested by the last step
     int* progress; int nsteps;       // rows finished so far (SYNC), number of steps
+    const int* abort_flag;           // set by any wait of the call that has run out
 };
 
 // End of a step: the per-frame barrier and, every PUBLISH steps, the progress counter.  Stores
@@ -897,7 +916,10 @@ __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
         else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
     }
     lds_barrier();
-    if (pub && threadIdx.x == 0) store_agent(cur.progress, last ? i + 2 : i + 2 - PUBLISH);
+    // (not after a wait of this call has run out -- the loader wave's for a strip of the gather, for
+    // one: rows computed from then on may be built on scores that were not there yet, and whoever waits
+    // for them must run into its own limit and write NaN rather than use them)
+    if (pub && threadIdx.x == 0 && !load_agent(cur.abort_flag)) store_agent(cur.progress, last ? i + 2 : i + 2 - PUBLISH);
 }
 
 // One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
@@ -994,6 +1016,7 @@ __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m,
     cur.c = 0.0;
     cur.pending = false;
     cur.progress = a.sync + SYNC_HDR + 2 * b + dir;
+    cur.abort_flag = a.sync;
     cur.nsteps = L - 1;
     if (SYNC) wait_stores();
     lds_barrier();
@@ -1214,6 +1237,8 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
 // LDS of a recursion workgroup, in floats: two emission rows, two state vectors (of doubles in
 // the uncapped instance, see recurse_step), per-wave minima / reduction scratch, a flag.
 constexpr int REC_LDS_FLOATS_F32 = 2 * D_MAX + 2 * (S_MAX + 16) + 32 + 8;
+static_assert(DENSE_F64_STATES >= 4 * REC_THREADS_DENSE, "the second size class of the dense instance fits in double");
+static_assert(2 * (DENSE_F64_STATES + 16) * 2 <= 2 * (S_MAX + 16), "two double vectors fit the float instance's state area");
 constexpr int REC_LDS_FLOATS_F64 = 2 * D_MAX + 4 * (S_MAX + 16) + 32 + 8;
 
 // the compute threads' part for one state type; the loader waves do not depend on it
@@ -1222,14 +1247,15 @@ constexpr int REC_LDS_FLOATS_F64 = 2 * D_MAX + 4 * (S_MAX + 16) + 32 + 8;
 // MANY: the same for the larger classes and the table-driven fallback
 template <bool SYNC, int T_, typename ST, bool ONE, bool MANY = true>
 __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int cls,
-                                                 ST* st0, ST* st1, const float* am0, const float* am1, float* wmin) {
+                                                 ST* st0, ST* st1, const float* am0, const float* am1, float* wmin,
+                                                 const int scap_big = S_MAX) {
     const int K = dir ? m.Kout : m.Kin;
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
     // (No six-edge specialisation for double: it is the rare case.)
     constexpr bool F32 = sizeof(ST) == 4;
     if (MANY && K > KMAX) {
-        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
+        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, scap_big);
     } else if (ONE && cls == 1) {
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
@@ -1244,7 +1270,7 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
         else if (K <= 4) recurse_compute<SYNC, T_, 4, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, 4 * T_);
     } else {
-        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, S_MAX);
+        recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, scap_big);
     }
 }
 
@@ -1283,8 +1309,7 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
         // the sequence's share of the compact emission table is unused on this path: room for the
         // two double-precision working vectors of each direction, unless T is tiny
         const long long goff = slot_off(m.edge_begin, b);
-        const long long room = (long long)a.T * (slot_off(m.edge_begin + m.n_edges, b + 1) - goff) / 2;      // in doubles
-        if (room >= 4LL * m.SP)
+        if (generic_recurse_f64_room(m, b, a.T))
             generic_recurse_f64<SYNC>(a.gen, m, b, dir, a.T, rows, offs, progress, wmin,
                                       (double*)(a.gtab_rw + (size_t)a.T * goff) + (size_t)dir * 2 * m.SP);
         else
@@ -1312,12 +1337,20 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // frames): batches of more than 128 CTC automata of 110-150 labels over 760-900 frames came out at
     // 8.7e-5 to 9.3e-5 in float.
     const bool small_tight = cls == 1 && m.SP <= 256 && m.L < 4LL * m.S;
-    const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > 1024);
+    const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES);
     // (there double costs half of the recursion time again, so only from 384 frames on, where the
     // rounding of float has had time to add up; but for every sequence with one state per thread)
-    if (DENSE && cls == 1 && ((m.L < 4LL * m.S && m.L >= 384) || m.L > 1024) && (dir ? m.Kout : m.Kin) <= KMAX) {
+    if (DENSE && cls == 1 && m.L >= 384 && (dir ? m.Kout : m.Kin) <= KMAX) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true, false>(a, m, b, dir, cls, st0, st0 + (T_ + 16), amr[0], amr[1], wmin);
+    } else if (DENSE && cls >= 2 && (5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES)) {
+        // The state area of this instance holds two double vectors of DENSE_F64_STATES + 16 entries (the
+        // preparation sends larger sequences of such batches to the general path, see dense_f64_limit).
+        // The register cap makes this slow; it is the rare case (hundreds of sequences with thousands
+        // of states each and barely more frames than states, or more than I6_FLOAT_FRAMES frames).
+        double* st0 = (double*)stf;
+        recurse_dispatch<SYNC, T_, double, false, true>(a, m, b, dir, cls, st0, st0 + (DENSE_F64_STATES + 16), amr[0], amr[1], wmin,
+                                                        DENSE_F64_STATES);
     } else if (wide) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true>(a, m, b, dir, cls, st0, st0 + (S_MAX + 16), amr[0], amr[1], wmin);
@@ -2384,6 +2417,15 @@ int runs_beside(Pipeline& p, hipStream_t s, bool* yes) {
     return I6FBW_OK;
 }
 
+// A hand-off timeout means that kernels which should have run side by side did not: the answers
+// cached per stream are dropped, and the next large call on a stream checks again.
+void forget_stream_checks() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lock(g_pipe[dev].mu);
+    g_pipe[dev].checked.clear();
+}
+
 // Stage timing: event pairs around every launch of a stage, on the stream it runs on.
 struct Profile {
     std::atomic<bool> on{false};
@@ -2421,7 +2463,6 @@ size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size
 constexpr int COMB_TILE_W = 12288;     // floats of a row that go through LDS at a time when the row does not fit: three workgroups per unit
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
-std::atomic<int> g_no_band{0};      // see i6fbw_set_band
 std::atomic<int> g_overlap_mode{[] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
@@ -2433,6 +2474,8 @@ std::atomic<int> g_writer_mode{[] {
     const char* e = getenv("I6FBW_DENSE_WRITER");
     return e ? (e[0] == 'r' ? 0 : 1) : -1;
 }()};
+
+std::atomic<int> g_last_writer{0};     // writer of the most recent i6fbw_run of the process: 0 rows, 1 flat spans
 
 // Status reports that travel to the host without a wait: per device a ring of pinned {code, seq}
 // slots, each with the event that follows its copy on the caller's stream.
@@ -2467,7 +2510,7 @@ std::atomic<int> g_status_mode{[] {
     return (a && a[0] == '1') ? 0 : 2;
 }()};
 
-int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int input_flags,
              const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
              int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
              int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
@@ -2492,12 +2535,12 @@ int i6fbw_run(const float* am, int64_t am_stride_t, int64_t am_stride_b, const i
                              workspace, workspace_bytes, stream_);
 }
 
-int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+int i6fbw_run_strided(const float* am, int64_t am_stride_t, int64_t am_stride_b, int input_flags,
                       const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
                       int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
                       int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
                       void* workspace, size_t workspace_bytes, void* stream_) {
-    return run_impl(am, am_stride_t, am_stride_b, scores_are_log_probs, edges, edge_row_stride, weights, start_end,
+    return run_impl(am, am_stride_t, am_stride_b, input_flags, edges, edge_row_stride, weights, start_end,
                     se_row_stride, seq_lens, T, B, F, E, n_states, out_mode, out, out_stride_t, out_stride_b, sum_output,
                     workspace, workspace_bytes, stream_, false);
 }
@@ -2528,7 +2571,7 @@ namespace {
 // Body of i6fbw_run_strided and i6fbw_run_static.  static_call: the workspace is the device's
 // built-in buffer, and nothing may be allocated or created -- no library streams or events, no
 // stage timers: the stages run one after the other on the caller's stream.
-int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int input_flags,
              const int32_t* edges, int64_t edge_row_stride, const float* weights, const int32_t* start_end,
              int64_t se_row_stride, const int32_t* seq_lens, int T, int B, int F, int E, int n_states,
              int out_mode, float* out, int64_t out_stride_t, int64_t out_stride_b, float* sum_output,
@@ -2537,6 +2580,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     if (!am || !start_end || !seq_lens || !out || !sum_output || (!workspace && !static_call)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (E > 0 && (!edges || !weights)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB && out_mode != I6FBW_OUT_NEG_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
+    if (input_flags & ~(I6FBW_IN_LOG_PROBS | I6FBW_IN_ALL_FRAMES)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_stride_t < 0 || out_stride_b < 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
@@ -2598,7 +2642,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
-    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = g_no_band; pa.force_generic = f_too_large ? 1 : 0;
+    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = (input_flags & I6FBW_IN_ALL_FRAMES) ? 1 : 0; pa.dense = (2 * B > P.n_cu && T <= 4096) ? 1 : 0; pa.force_generic = f_too_large ? 1 : 0;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx); pa.renum = (int2*)(ws + l.renum);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
@@ -2606,10 +2650,11 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     GatherArgs ga;
     ga.am = am; ga.st_t = am_stride_t; ga.st_b = am_stride_b; ga.T = T; ga.B = B;
     ga.meta = meta; ga.demis = pa.demis; ga.tband = pa.tband; ga.gtab = (float*)(ws + l.gtab); ga.sync = sync;
-    ga.scale = scores_are_log_probs ? -LOG2E : LOG2E; ga.ascending = 0;
+    ga.scale = (input_flags & I6FBW_IN_LOG_PROBS) ? -LOG2E : LOG2E; ga.ascending = 0;
     GenArgs gen;
-    gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = scores_are_log_probs ? -1.f : 1.f;
+    gen.am = am; gen.st_t = am_stride_t; gen.st_b = am_stride_b; gen.sign = (input_flags & I6FBW_IN_LOG_PROBS) ? -1.f : 1.f;
     gen.edges = edges; gen.edge_stride = edge_row_stride; gen.weights = weights; gen.eidx = pa.eidx; gen.renum = pa.renum;
+    gen.all_frames = (input_flags & I6FBW_IN_ALL_FRAMES) ? 1 : 0;
     RecArgs ra;
     ra.gen = gen;
     ra.T = T; ra.B = B; ra.prep_wgs = 3 * B; ra.meta = meta; ra.ellA = pa.ellA; ra.ellB = pa.ellB; ra.gtab = ga.gtab; ra.gtab_rw = ga.gtab;
@@ -2650,6 +2695,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
         if (flat_grid > 0x7fffffffLL || (long long)TC * rows * F >= (1LL << 31) - FLAT_W) flat = false;
     }
     ca.direct_only = flat ? 1 : 0;
+    g_last_writer = flat ? 1 : 0;
 
     {
         // the scan also clears the header of the hand-off area, so it runs even without edges
@@ -2670,7 +2716,19 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
         HIP_TRY(hipEventRecord(P.doneR, sR));
         return I6FBW_OK;
     };
+    // Whatever way this function is left once the library streams have been given work: the caller's
+    // stream waits for them, so that nothing enqueued on it afterwards (the release of a torch-owned
+    // workspace, say) can overtake kernels that still use the workspace.
+    struct JoinGuard {
+        Pipeline& P; hipStream_t s; bool armed = false, joined = false;
+        ~JoinGuard() {
+            if (!armed || joined) return;
+            if (hipEventRecord(P.doneP, P.sP) == hipSuccess) (void)hipStreamWaitEvent(s, P.doneP, 0);
+            if (hipEventRecord(P.doneR, P.sR) == hipSuccess) (void)hipStreamWaitEvent(s, P.doneR, 0);
+        }
+    } join_guard{P, s};
     if (overlap) {
+        join_guard.armed = true;
         // The library streams are released when the scan is done, i.e. while the preparation's
         // workgroups are being placed.  The recursion's 2B large workgroups need nine free wave
         // slots on one compute unit each and find them while the machine is still almost empty;
@@ -2749,6 +2807,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int scor
     // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
+    join_guard.joined = true;
     return I6FBW_OK;
 }
 }  // namespace
@@ -2777,6 +2836,7 @@ int i6fbw_read_status(const void* workspace, int B, void* stream, int* code, int
     memcpy(&aborted, host + flag_at, sizeof(int));
     const SeqMeta* meta = (const SeqMeta*)host;
     *code = aborted ? I6FBW_ERR_TIMEOUT : I6FBW_OK; *seq = -1;
+    if (aborted) forget_stream_checks();
     for (int b = 0; b < B; b++) {
         // positive values mark sequences that took the general path
         const int c = meta[b].err < 0 ? meta[b].err : (meta[b].errA < 0 ? meta[b].errA : (meta[b].errB < 0 ? meta[b].errB : 0));
@@ -2825,6 +2885,7 @@ int i6fbw_poll_status(int wait, int* code, int* seq) {
         if (!status_collect(r, (r.next + k) % StatusRing::SLOTS, wait != 0)) break;
     *code = r.held_code; *seq = r.held_seq;
     r.held_code = I6FBW_OK; r.held_seq = -1;
+    if (*code == I6FBW_ERR_TIMEOUT) g_pipe[dev].checked.clear();      // (this device's lock is held)
     return I6FBW_OK;
 }
 
@@ -2844,11 +2905,7 @@ const char* i6fbw_strerror(int code) {
         case I6FBW_ERR_INVALID_ARGUMENT: return "invalid argument";
         case I6FBW_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
         case I6FBW_ERR_LAUNCH: return "HIP call failed";
-        case I6FBW_ERR_F_TOO_LARGE: return "number of emission classes F exceeds the supported maximum";
-        case I6FBW_ERR_SEQ_TOO_MANY_EDGES: return "a sequence has more edges than supported (8192)";
-        case I6FBW_ERR_SEQ_SPARSE_STATES: return "state ids of a sequence span more than 2*edges+2 ids (not reported any more)";
-        case I6FBW_ERR_SEQ_DEGREE: return "a state has more than 8 incoming or outgoing edges";
-        case I6FBW_ERR_SEQ_TOO_LARGE: return "a sequence has more than 4096 states or distinct emissions";
+        case I6FBW_ERR_SEQ_TOO_LARGE: return "best path: a sequence on the general path does not fit its share of the workspace";
         case I6FBW_ERR_BAD_INDEX: return "sequence, emission or state index out of range";
         case I6FBW_ERR_TIMEOUT: return "a kernel gave up waiting for another stage of the same call";
         case I6FBW_ERR_STATIC_WORKSPACE: return "the problem needs more workspace than the built-in buffer of i6fbw_run_static holds (32 MiB)";
@@ -2856,7 +2913,14 @@ const char* i6fbw_strerror(int code) {
     }
 }
 
+int i6fbw_set_spin_limit(int polls) {
+    const int v = polls > 0 ? polls : SPIN_LIMIT;
+    HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_spin_limit), &v, sizeof(int)));
+    return I6FBW_OK;
+}
+
 void i6fbw_set_dense_writer(int mode) { g_writer_mode = mode < 0 ? -1 : (mode ? 1 : 0); }
+int i6fbw_last_dense_writer(void) { return g_last_writer.load(); }
 
 void i6fbw_set_overlap(int mode) {
     std::lock_guard<std::mutex> lock(g_mutex);
@@ -2867,11 +2931,6 @@ void i6fbw_set_overlap(int mode) {
 int i6fbw_debug_trace(void* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_trace), sizeof(unsigned long long) * n); }
 int i6fbw_debug_trace_set(const void* host, int n) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), host, sizeof(unsigned long long) * n); }
 #endif
-
-void i6fbw_set_band(int on) {
-    std::lock_guard<std::mutex> lock(g_mutex);
-    g_no_band = on ? 0 : 1;
-}
 
 // Text dumps of fbw_op.cu:155-224.  Host code: device-to-host copies and file output.
 int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32_t* start_end, int64_t se_row_stride,
@@ -2886,29 +2945,58 @@ int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32
     HIP_TRY(hipMemcpy(se.data(), start_end, sizeof(int32_t) * B, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(se.data() + B, start_end + se_row_stride, sizeof(int32_t) * B, hipMemcpyDeviceToHost));
     std::vector<float> rows;
+    std::vector<double> rows64;
+    std::vector<int2> renum;
     for (int b = 0; b < B; b++) {
         const std::string name = std::string(directory) + "/alignment.dump." + std::to_string(batch_idx) + "." + std::to_string(b);
         FILE* f = fopen(name.c_str(), "w");
         if (!f) return I6FBW_ERR_INVALID_ARGUMENT;
         const SeqMeta& m = meta[b];
-        const bool ok = !(m.err || m.errA || m.errB) && !(m.pad & 2);      // (no dump for renumbered state ids)
+        const bool ok = m.err >= 0 && m.errA >= 0 && m.errB >= 0;   // (a sequence with a reported problem has no rows)
+        const bool general = ok && (m.err > 0 || m.errA > 0 || m.errB > 0);
         const long long first = se[b], last = se[B + b];           // the reference walks the ids start..end
         // frame 0 is written even for an empty sequence (fbw_op.cu:177); it holds the start state only
         const int frames = !ok ? 0 : (m.L > 0 && m.n_edges > 0 ? m.L : 1);
         const bool have_rows = ok && m.L > 0 && m.n_edges > 0;
+        // a sequence on the general path keeps its rows in double where they fit, and in natural-log units
+        const long long soff = state_off(m.edge_begin, b);
+        const long long share = state_off((long long)m.edge_begin + m.n_edges, b + 1) - soff;
+        const long long groom = (long long)T * (slot_off((long long)m.edge_begin + m.n_edges, b + 1) - slot_off(m.edge_begin, b)) / 2;
+        const bool r64 = general && 2LL * m.SP <= share && groom >= 4LL * m.SP;
+        const float unit = general ? 1.f : LN2;
         if (have_rows) {
-            rows.resize((size_t)m.L * m.SP);
-            const float* src = (const float*)((const char*)workspace + l.alpha) + (size_t)T * state_off(m.edge_begin, b);
-            if (hipMemcpy(rows.data(), src, sizeof(float) * rows.size(), hipMemcpyDeviceToHost) != hipSuccess) { fclose(f); return I6FBW_ERR_LAUNCH; }
+            const char* src = (const char*)workspace + l.alpha + sizeof(float) * (size_t)T * soff;
+            hipError_t e;
+            if (r64) { rows64.resize((size_t)m.L * m.SP); e = hipMemcpy(rows64.data(), src, sizeof(double) * rows64.size(), hipMemcpyDeviceToHost); }
+            else { rows.resize((size_t)m.L * m.SP); e = hipMemcpy(rows.data(), src, sizeof(float) * rows.size(), hipMemcpyDeviceToHost); }
+            if (e != hipSuccess) { g_last_hip_error = e; fclose(f); return I6FBW_ERR_LAUNCH; }
+            if (m.pad & 2) {
+                // state ids spread over a wide range: their numbers within the sequence sit in an open-addressing table
+                renum.resize(renum_capacity(m.n_edges));
+                e = hipMemcpy(renum.data(), (const char*)workspace + l.renum + sizeof(int2) * 2 * (size_t)soff, sizeof(int2) * renum.size(),
+                              hipMemcpyDeviceToHost);
+                if (e != hipSuccess) { g_last_hip_error = e; fclose(f); return I6FBW_ERR_LAUNCH; }
+            }
         }
+        // number of state id sid within the sequence, -1 if the sequence does not name it
+        auto local = [&](long long sid) -> long long {
+            if (!(m.pad & 2)) { const long long loc = sid - m.state_min; return loc >= 0 && loc < m.S ? loc : -1; }
+            const unsigned cap = (unsigned)renum.size();
+            unsigned h = renum_home((int)sid, cap);
+            while (true) {
+                if (renum[h].x == (int)sid + 1) return renum[h].y;
+                if (renum[h].x == 0) return -1;
+                h = h + 1 == cap ? 0 : h + 1;
+            }
+        };
         for (int t = 0; t < frames; t++) {
-            // value of state id s in natural-log units (rows are stored in units of log 2, relative
-            // to an offset that cancels in the normalisation)
+            // value of state id s in natural-log units (rows of the fast kernels are stored in units of
+            // log 2; all rows are relative to an offset that cancels in the normalisation)
             auto value = [&](long long sid) -> float {
-                const long long loc = sid - m.state_min;
                 if (!have_rows) return sid == first ? 0.f : INFINITY;
-                if (loc < 0 || loc >= m.S) return INFINITY;
-                return rows[(size_t)t * m.SP + loc] * LN2;
+                const long long loc = local(sid);
+                if (loc < 0) return INFINITY;
+                return r64 ? (float)rows64[(size_t)t * m.SP + loc] : rows[(size_t)t * m.SP + loc] * unit;
             };
             float sum = INFINITY;
             for (long long sid = first; sid <= last; sid++) {

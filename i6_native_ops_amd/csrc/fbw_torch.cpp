@@ -3,6 +3,7 @@
 // seq_lens, num_states, debug_options=DebugOptions()) -> [out (T,B,F), sum_output (T,B)].
 // torch is used for device memory and the current stream only; all arithmetic is behind the
 // C ABI declared in include/i6fbw.h.
+#include <atomic>
 #include <cstdlib>
 #include <vector>
 
@@ -77,14 +78,13 @@ static std::vector<torch::Tensor> run(torch::Tensor& am_scores, torch::Tensor& e
     // the alignment dump needs the forward scores of every state, also of those that cannot reach
     // the end state any more
     const bool all_scores = dump && dump->dump_alignment;
-    if (all_scores) i6fbw_set_band(0);
-    rc = i6fbw_run_strided(am_scores.data_ptr<float>(), am_scores.stride(dt), am_scores.stride(db), fused ? 1 : 0,
+    const int input_flags = (fused ? I6FBW_IN_LOG_PROBS : 0) | (all_scores ? I6FBW_IN_ALL_FRAMES : 0);
+    rc = i6fbw_run_strided(am_scores.data_ptr<float>(), am_scores.stride(dt), am_scores.stride(db), input_flags,
                            edges.data_ptr<int32_t>(), edges.stride(0), weights.data_ptr<float>(),
                            start_end_states.data_ptr<int32_t>(), start_end_states.stride(0),
                            seq_lens.data_ptr<int32_t>(), T, B, F, E, (int)num_states, out_mode, out.data_ptr<float>(),
                            out.stride(dt), out.stride(db), sum_output.data_ptr<float>(), workspace.data_ptr(), ws_bytes,
                            (void*)stream);
-    if (all_scores) i6fbw_set_band(1);
     TORCH_CHECK(rc == I6FBW_OK, "NativeOp: fbw: ", i6fbw_strerror(rc), " ", i6fbw_last_hip_error());
     // a dump reads the workspace on the host anyway: such a call waits for its own status
     if (dump && i6fbw_get_status_mode() == 2) {
@@ -114,7 +114,7 @@ std::vector<torch::Tensor> fbw(torch::Tensor& am_scores, torch::Tensor& edges, t
                                torch::Tensor& start_end_states, torch::Tensor& seq_lens, unsigned num_states,
                                DebugOptions debug_options = DebugOptions()) {
     // calls are numbered as in the reference (fbw_op.cu:246,390); every dump_every-th one is dumped
-    static unsigned batch_idx = 0u;
+    static std::atomic<unsigned> batch_idx{0u};
     const unsigned idx = batch_idx++;
     const bool dump_now = (debug_options.dump_alignment || debug_options.dump_output) && debug_options.dump_every > 0u &&
                           idx % debug_options.dump_every == 0u;

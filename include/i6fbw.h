@@ -27,15 +27,9 @@ enum {
     I6FBW_ERR_LAUNCH = -3,             /* a HIP launch failed; see i6fbw_last_hip_error() */
     /* Sequences beyond the capacity of the fast kernels (more than 8192 edges, 4096 states or 4096
        distinct emissions in one sequence, more than 15 edges into or out of a state, F beyond
-       131 072) are not refused: they take a general path
-       that has no such limits and runs at a fraction of the speed.  The size codes remain for the
-       one case that path cannot hold either. */
-    I6FBW_ERR_F_TOO_LARGE = -4,           /* not returned any more */
-    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,   /* not reported any more */
-    I6FBW_ERR_SEQ_SPARSE_STATES = -11,    /* not reported any more: a sequence whose state ids span more than
-                                             2*edges+2 ids gets dense numbers for its states on the device */
-    I6FBW_ERR_SEQ_DEGREE = -12,           /* not reported any more */
-    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side, i6fbw_viterbi: values and back-pointers of a sequence on the
+       131 072) are not refused: they take a general path that has no such limits and runs at a
+       fraction of the speed. */
+    I6FBW_ERR_SEQ_TOO_LARGE = -13,        /* device-side, i6fbw_viterbi only: values and back-pointers of a sequence on the
                                              general path do not fit its share of the workspace (T < 2*edges+16 with
                                              state ids spread over nearly 2*edges ids) */
     I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
@@ -104,12 +98,16 @@ int i6fbw_run(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
  * fbw_loss (fbw/__init__.py:47-68) and wants the gradient in the same layout without the
  * reference wrapper's dense passes (neg, transpose().contiguous(), neg, exp and their autograd
  * inverses: fbw/__init__.py:43,66):
- *   scores_are_log_probs  0: am_scores holds -log p (as for i6fbw_run), 1: it holds log p
+ *   input_flags           I6FBW_IN_LOG_PROBS: am_scores holds log p instead of -log p;
+ *                         I6FBW_IN_ALL_FRAMES: gather the score of every (frame, emission) pair, also where
+ *                         the emission cannot carry mass (slower, same outputs; i6fbw_dump_alignment needs
+ *                         the forward scores of such states).  Per call: nothing process-wide is touched.
  *   out_stride_t/_b       element strides of out over frames / sequences (innermost stride 1);
  *                         rows may overlap nothing else and need not be aligned
  * i6fbw_run(...) is i6fbw_run_strided(..., 0, ..., out, B*F, F, ...).
  */
-int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b, int scores_are_log_probs,
+enum { I6FBW_IN_LOG_PROBS = 1, I6FBW_IN_ALL_FRAMES = 2 };
+int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b, int input_flags,
                       const int32_t* edges, int64_t edge_row_stride,
                       const float* weights,
                       const int32_t* start_end, int64_t se_row_stride,
@@ -219,6 +217,15 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
 void i6fbw_set_overlap(int mode);
 
 /*
+ * Kernels of the overlapped schedule that wait for another kernel of the same call poll at most
+ * `polls` times (default 2^20, restored by polls <= 0) before they give up: the call then reports
+ * I6FBW_ERR_TIMEOUT and the rows that could not be computed hold NaN.  Device-wide for the current
+ * device; it exists so that a test can force that path from the host (polls = 1) while every kernel
+ * still runs to its normal end.  No counterpart in the reference.
+ */
+int i6fbw_set_spin_limit(int polls);
+
+/*
  * Chooses how i6fbw_run writes the dense (T, B, F) tensor: 0 row by row (one workgroup per strip of
  * frames of a sequence builds each row in LDS and streams it out), 1 in flat 128-byte-aligned spans
  * fed from compact per-frame posteriors wherever the output is one contiguous block ((T, B, F) or
@@ -228,6 +235,9 @@ void i6fbw_set_overlap(int mode);
  * atomics into a pre-filled tensor).
  */
 void i6fbw_set_dense_writer(int mode);
+/* Which writer the most recent i6fbw_run / i6fbw_run_strided of the process used: 0 rows, 1 flat spans
+ * (for benchmarks that price the kernel that wrote the tensor). */
+int i6fbw_last_dense_writer(void);
 
 /*
  * Device-side construction of the automaton arrays for two common topologies.  No counterpart in
@@ -277,18 +287,15 @@ int i6fbw_build_hmm_fsa(const int32_t* labels, int64_t label_row_stride, const i
  * i6fbw_dump_alignment: file alignment.dump.<batch_idx>.<seq>, a line "t (state - start) value"
  * for the states start..end of the sequence, where value = forward score of the state before
  * frame t minus the log-sum over those states, if <= pruning, as write_alignment_to_file
- * (fbw_op.cu:155-197).  It reads the forward rows of the last i6fbw_run on `workspace`; call
- * i6fbw_set_band(0) before that run, otherwise states that cannot reach the end state in the
- * remaining frames are missing (their scores are never computed), and i6fbw_set_band(1) after it.
+ * (fbw_op.cu:155-197).  It reads the forward rows of the last i6fbw_run_strided on `workspace`; make
+ * that call with I6FBW_IN_ALL_FRAMES, otherwise states that cannot reach the end state in the
+ * remaining frames are missing (their scores are never computed).
  * Sequences whose length is outside [1, T] have no forward rows: frame 0 alone is written.
  */
 int i6fbw_dump_output(const float* out, int64_t out_stride_t, int64_t out_stride_b, const int32_t* seq_lens,
                       int T, int B, int F, float pruning, unsigned batch_idx, const char* directory, void* stream);
 int i6fbw_dump_alignment(const void* workspace, int T, int B, int E, const int32_t* start_end, int64_t se_row_stride,
                          float pruning, unsigned batch_idx, const char* directory, void* stream);
-/* 1 (default): scores outside the frames in which an emission can carry mass are not gathered;
- * 0: all are (slower, same outputs; needed for i6fbw_dump_alignment).  Process-wide. */
-void i6fbw_set_band(int on);
 
 /* Text for a status code. */
 const char* i6fbw_strerror(int code);

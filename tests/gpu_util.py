@@ -21,12 +21,19 @@ class DeviceProblem:
         self.ws_bytes = cabi.workspace_size(self.T, self.B, self.F, self.E, self.n_states)
         self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
 
-    def run(self, out_mode=cabi.OUT_NEG_LOG, check=True):
+    def run(self, out_mode=cabi.OUT_NEG_LOG, check=True, input_flags=None):
         stream = torch.cuda.current_stream().cuda_stream
-        cabi.run(self.am.data_ptr(), self.am.stride(0), self.am.stride(1), self.edges.data_ptr(),
-                 self.edges.stride(0) if self.E > 0 else 0, self.weights.data_ptr(), self.start_end.data_ptr(),
-                 self.start_end.stride(0), self.seq_lens.data_ptr(), self.T, self.B, self.F, self.E, self.n_states,
-                 out_mode, self.out.data_ptr(), self.loss.data_ptr(), self.ws.data_ptr(), self.ws_bytes, stream)
+        if input_flags is None:
+            cabi.run(self.am.data_ptr(), self.am.stride(0), self.am.stride(1), self.edges.data_ptr(),
+                     self.edges.stride(0) if self.E > 0 else 0, self.weights.data_ptr(), self.start_end.data_ptr(),
+                     self.start_end.stride(0), self.seq_lens.data_ptr(), self.T, self.B, self.F, self.E, self.n_states,
+                     out_mode, self.out.data_ptr(), self.loss.data_ptr(), self.ws.data_ptr(), self.ws_bytes, stream)
+        else:
+            cabi.run_strided(self.am.data_ptr(), self.am.stride(0), self.am.stride(1), input_flags, self.edges.data_ptr(),
+                             self.edges.stride(0) if self.E > 0 else 0, self.weights.data_ptr(), self.start_end.data_ptr(),
+                             self.start_end.stride(0), self.seq_lens.data_ptr(), self.T, self.B, self.F, self.E,
+                             self.n_states, out_mode, self.out.data_ptr(), self.out.stride(0), self.out.stride(1),
+                             self.loss.data_ptr(), self.ws.data_ptr(), self.ws_bytes, stream)
         if check:
             code, seq = cabi.read_status(self.ws.data_ptr(), self.B, stream)
             if code != 0:

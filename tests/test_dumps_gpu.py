@@ -122,12 +122,8 @@ def test_dump_through_the_c_abi(in_tmp, oracle):
     from i6_native_ops_amd.fbw.workloads import make_workload
     from tests.gpu_util import DeviceProblem
     wl = make_workload("tiny")
-    cabi.set_band(False)
-    try:
-        P = DeviceProblem(wl.am_scores, wl.edges, wl.weights, wl.start_end_states, wl.seq_lens, wl.n_states)
-        out, _ = P.run(cabi.OUT_NEG_LOG)
-    finally:
-        cabi.set_band(True)
+    P = DeviceProblem(wl.am_scores, wl.edges, wl.weights, wl.start_end_states, wl.seq_lens, wl.n_states)
+    out, _ = P.run(cabi.OUT_NEG_LOG, input_flags=cabi.IN_ALL_FRAMES)
     stream = torch.cuda.current_stream().cuda_stream
     cabi.dump_alignment(P.ws.data_ptr(), P.T, P.B, P.E, P.start_end.data_ptr(), P.start_end.stride(0), 1e30, 7, ".", stream)
     cabi.dump_output(out.data_ptr(), out.stride(0), out.stride(1), P.seq_lens.data_ptr(), P.T, P.B, P.F, 1e30, 7, ".", stream)
@@ -142,3 +138,57 @@ def test_dump_through_the_c_abi(in_tmp, oracle):
         finite = [(t, e) for t in range(L) for e in range(wl.F) if np.isfinite(want_out[t, b, e])]
         assert [(t, e) for t, e, _ in rows] == finite
         np.testing.assert_allclose([v for *_, v in rows], [want_out[t, b, e] for t, e in finite], atol=2e-4, rtol=1e-4)
+
+
+def _forward_rows(am_b, frm, to, emis, w, start, n_states, L):
+    """-log forward scores of every state id before each of the L frames (plain numpy, fbw_op.cu:318-333)"""
+    neg = np.full(n_states, -np.inf)
+    neg[start] = 0.0
+    rows = [-neg]
+    for t in range(L - 1):
+        cand = neg[frm] - w - am_b[t, emis].astype(np.float64)
+        nxt = np.full(n_states, -np.inf)
+        np.logaddexp.at(nxt, to, cand)
+        neg = nxt
+        rows.append(-neg)
+    return rows
+
+
+@pytest.mark.parametrize("case", ["general_path", "spread_ids"])
+def test_alignment_dump_of_sequences_off_the_common_path(in_tmp, case):
+    """A sequence too large for the fast kernels (more than 8192 edges: general path, rows in double) and one
+    whose state ids are spread over a wide range (renumbered on the device): the dump lists the normalised
+    forward scores of the ids start..end as for any other sequence (fbw_op.cu:155-196)."""
+    from i6_native_ops_amd import cabi
+    from i6_native_ops_amd.fbw.workloads import make_workload
+    from tests.gpu_util import DeviceProblem
+    from tests.helpers import spread_state_ids
+    if case == "general_path":
+        wl = make_workload("cart", T=40, B=2, F=50, n_labels=(1400, 1400))       # 8400 edges per sequence
+        edges, start_end, n_states = wl.edges, wl.start_end_states, wl.n_states
+    else:
+        wl = make_workload("cart", T=40, B=2, F=50, n_labels=(6, 9))
+        edges, start_end, n_states = spread_state_ids(wl.edges, wl.start_end_states, wl.n_states, how="stride")
+    wl.seq_lens[:] = [40, 33]
+    P = DeviceProblem(wl.am_scores, edges, wl.weights, start_end, wl.seq_lens, n_states)
+    P.run(cabi.OUT_NEG_LOG, input_flags=cabi.IN_ALL_FRAMES)
+    stream = torch.cuda.current_stream().cuda_stream
+    pruning = 30.0
+    cabi.dump_alignment(P.ws.data_ptr(), P.T, P.B, P.E, P.start_end.data_ptr(), P.start_end.stride(0), pruning, 3, ".", stream)
+    for b in range(wl.B):
+        L = int(wl.seq_lens[b])
+        sel = edges[3] == b
+        first, last = int(start_end[0, b]), int(start_end[1, b])
+        rows = _forward_rows(wl.am_scores[:, b], edges[0, sel], edges[1, sel], edges[2, sel], wl.weights[sel].astype(np.float64),
+                             first, n_states, L)
+        got = parse(f"alignment.dump.3.{b}")
+        assert {t for t, *_ in got} == set(range(L))
+        lo, hi = min(first, last), max(first, last)
+        for t in range(L):
+            r = rows[t][lo:hi + 1] if first <= last else rows[t][0:0]
+            z = -np.logaddexp.reduce(-r)
+            want = {i: float(v - z) for i, v in enumerate(r) if v - z <= pruning - 1e-3}
+            have = {i: v for tt, i, v in got if tt == t}
+            assert set(want) <= set(have)
+            for i, v in want.items():
+                assert have[i] == pytest.approx(v, abs=2e-4, rel=1e-5)

@@ -1,0 +1,138 @@
+"""Seeded randomised parity sweep of i6fbw_run against the fp64 oracle, through the C ABI.
+
+The recursion keeps the state vector of a sequence in float or in double depending on its shape
+(frames per state, length, batch size: see recurse_workgroup).  This sweep pins the bar -- loss
+relative error <= 1e-5, posterior absolute error <= 1e-4 -- on random shapes of all three automaton
+families, under both schedules, and on shapes placed on either side of every one of those
+decisions: 1024 / 1025 frames, five states for three frames, 256 states with four frames each,
+and, for batches of more than 128 sequences (the recursion instance of which two workgroups share a
+compute unit), 383 / 384 frames, more than 1024 frames and more states than that instance has
+compute threads.  Every case is printed with its errors; the cases beyond the bar fail the test.
+"""
+import numpy as np
+import pytest
+
+from i6_native_ops_amd.fbw.workloads import make_workload
+from tests.helpers import posterior
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+POST_ATOL = 1e-4
+
+
+def chain_workload(kind, seed, T, B, F, n_labels, lens):
+    W = make_workload(kind, seed=seed, T=T, B=B, F=F, n_labels=n_labels)
+    lens = np.asarray(lens, dtype=np.int32)
+    W.seq_lens[:] = np.resize(lens, B)
+    return W
+
+
+def worst_errors(oracle, W, overlap):
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import run_cabi
+    args = (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    want_out, want_loss = oracle.fbw_oracle(*args, threads=16)
+    cabi.set_overlap(overlap)
+    try:
+        out, loss = run_cabi(*args, out_mode=cabi.OUT_PROB)
+    finally:
+        cabi.set_overlap(-1)
+    nz = want_loss != 0
+    assert (loss[~nz] == 0).all()
+    lerr = float(np.max(np.abs(loss[nz] - want_loss[nz]) / np.abs(want_loss[nz]))) if nz.any() else 0.0
+    perr = float(np.max(np.abs(out - posterior(want_out))))
+    return lerr, perr
+
+
+def check(oracle, W, overlap, what, failures):
+    lerr, perr = worst_errors(oracle, W, overlap)
+    print(f"{what}: loss {lerr:.2e} posterior {perr:.2e}", flush=True)
+    if not (lerr <= LOSS_RTOL and perr <= POST_ATOL):
+        failures.append(f"{what}: loss {lerr:.2e} posterior {perr:.2e}")
+    return perr
+
+
+# (family, labels, frames): states = 3 * labels + 1 for the chains, 2 * labels + 3 for ctc
+THRESHOLD_CASES = [
+    # 1024 / 1025 frames (longer sequences always run in double), relaxed alignment
+    ("cart", 100, 1024), ("cart", 100, 1025), ("ctc", 120, 1024), ("ctc", 120, 1025),
+    # five states for every three frames: 3 L = 5 S at S = 601, L = 1001.67
+    ("cart", 200, 1000), ("cart", 200, 1002), ("cart", 200, 1004), ("monophone", 150, 760),
+    # at most 256 states and fewer than four frames per state: S = 250 -> L = 1000
+    ("cart", 83, 998), ("cart", 83, 1000), ("cart", 83, 1003), ("cart", 85, 1000), ("ctc", 124, 1000), ("ctc", 126, 1000),
+    # 512 / 513 frames
+    ("ctc", 120, 512), ("ctc", 120, 513), ("ctc", 200, 512), ("cart", 60, 512), ("cart", 60, 513), ("ctc", 60, 500), ("ctc", 30, 512),
+    # tight: one frame per state and a little more
+    ("cart", 300, 905), ("cart", 300, 960), ("ctc", 400, 810), ("cart", 340, 1024),
+]
+
+
+@pytest.mark.parametrize("overlap", [0, 1], ids=["single_stream", "overlapped"])
+def test_shapes_next_to_the_precision_decisions(oracle, overlap):
+    worst, failures = 0.0, []
+    for i, (kind, n, L) in enumerate(THRESHOLD_CASES):
+        W = chain_workload(kind, 300 + i, T=L + 3, B=3, F=211, n_labels=(n, n), lens=[L, L - 1, L + 2])
+        worst = max(worst, check(oracle, W, overlap, f"{kind} labels={n} frames={L}", failures))
+    print("worst posterior error", worst)
+    assert not failures, failures
+
+
+# more than 128 sequences: the instance with 448 compute threads of which two share a compute unit
+DENSE_CASES = [
+    ("ctc", 48, 383), ("ctc", 48, 384), ("ctc", 48, 399), ("ctc", 100, 500), ("cart", 40, 383), ("cart", 40, 384),
+    ("ctc", 60, 1024), ("ctc", 60, 1025), ("cart", 120, 1100),
+    # more states than the instance has compute threads (several states per thread), short and long
+    ("cart", 160, 700), ("cart", 160, 1100), ("ctc", 300, 1100), ("cart", 330, 1030),
+]
+
+
+@pytest.mark.parametrize("overlap", [0, 1], ids=["single_stream", "overlapped"])
+def test_large_batches_next_to_the_precision_decisions(oracle, overlap):
+    worst, failures = 0.0, []
+    for i, (kind, n, L) in enumerate(DENSE_CASES):
+        W = chain_workload(kind, 500 + i, T=L + 2, B=130, F=97, n_labels=(n, n), lens=[L, L - 1, L + 1, L - 7])
+        worst = max(worst, check(oracle, W, overlap, f"B=130 {kind} labels={n} frames={L}", failures))
+    print("worst posterior error", worst)
+    assert not failures, failures
+
+
+def test_large_batch_with_one_sequence_beyond_the_double_capacity_of_its_instance(oracle):
+    """129 small sequences and one tight one of 2101 states in a batch of more than 128: the recursion instance
+    for such batches has room for 2032 states in double, so the preparation sends it to the general path."""
+    from tests.test_flat_writer_gpu import merge
+    T = 2150
+    small = make_workload("ctc", seed=71, T=T, B=129, F=97, n_labels=(20, 40))
+    big = make_workload("cart", seed=72, T=T, B=1, F=97, n_labels=(700, 700))
+    big.seq_lens[:] = T - 3
+    am, edges, weights, se, lens, n_states = merge([small, big])
+
+    class W:
+        pass
+    W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states = am, edges, weights, se, lens, n_states
+    failures = []
+    for overlap in (0, 1):
+        check(oracle, W, overlap, f"129 small + 1 of 2101 states, overlap={overlap}", failures)
+    assert not failures, failures
+
+
+def test_random_shapes(oracle):
+    """160 random cases: family, size, tightness of the alignment, edge order, batch size, schedule."""
+    rng = np.random.default_rng(20241)
+    worst, failures = 0.0, []
+    for case in range(160):
+        kind = ["cart", "ctc", "monophone"][int(rng.integers(0, 3))]
+        n = int(rng.choice([3, 10, 30, 80, 85, 150, 250, 340]))
+        states = 3 * n + 1 if kind != "ctc" else 2 * n + 3
+        tight = float(rng.choice([1.02, 1.2, 1.6, 1.7, 2.5, 3.9, 4.1, 8.0]))
+        L = int(min(2100, max(states + 1, states * tight)))
+        B = int(rng.choice([1, 2, 5, 9]))
+        F = int(rng.choice([40, 211, 600]))
+        lens = [max(states, L - int(x)) for x in rng.integers(0, 6, size=B)]
+        W = make_workload(kind, seed=1000 + case, T=L, B=B, F=F, n_labels=(max(1, n - 2), n),
+                          shuffle_edges=bool(rng.integers(0, 2)))
+        W.seq_lens[:] = np.asarray(lens, dtype=np.int32)
+        overlap = int(rng.integers(0, 2))
+        worst = max(worst, check(oracle, W, overlap, f"case {case}: {kind} labels<={n} frames={L} B={B} F={F} overlap={overlap}", failures))
+    print("worst posterior error", worst)
+    assert not failures, failures
