@@ -24,12 +24,15 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
-def build_lib():
-    _run([HIPCC, *HIP_FLAGS, "-shared", os.path.join(CSRC, "fbw_kernels.hip"), "-o", LIB])
-    return LIB
+def build_lib(out_root=PKG):
+    """libi6fbw.so into <out_root>/fbw (out_root: this package in the source tree, or its copy in a build tree)"""
+    lib = os.path.join(out_root, "fbw", "libi6fbw.so")
+    os.makedirs(os.path.dirname(lib), exist_ok=True)
+    _run([HIPCC, *HIP_FLAGS, "-shared", os.path.join(CSRC, "fbw_kernels.hip"), "-o", lib])
+    return lib
 
 
-def build_ext(name="fbw_core", source="fbw_torch.cpp", out_dir=None):
+def build_ext(name="fbw_core", source="fbw_torch.cpp", out_dir=None, lib_dir=None):
     import torch
     from torch.utils import cpp_extension
     inc = cpp_extension.include_paths()
@@ -40,19 +43,22 @@ def build_ext(name="fbw_core", source="fbw_torch.cpp", out_dir=None):
            "-I" + sysconfig.get_paths()["include"], "-I/opt/rocm/include"]
     cmd += ["-I" + p for p in inc]
     out_dir = out_dir or OUT
+    os.makedirs(out_dir, exist_ok=True)
     ext = os.path.join(out_dir, name + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
     cmd += [os.path.join(CSRC, source), "-o", ext,
-            "-L" + OUT, "-li6fbw", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
+            "-L" + (lib_dir or OUT), "-li6fbw", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
             "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
             "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,$ORIGIN/../fbw", "-Wl,-rpath," + torch_lib, "-Wl,-rpath,/opt/rocm/lib", "-Wno-attributes"]
     _run(cmd)
     return ext
 
 
-def build_all():
-    build_lib()
-    build_ext()
-    build_ext("fast_viterbi_core", "viterbi_torch.cpp", os.path.join(PKG, "fast_viterbi"))
+def build_all(out_root=PKG):
+    """Everything native, into the package directory out_root (default: in the source tree)."""
+    build_lib(out_root)
+    lib_dir = os.path.join(out_root, "fbw")
+    build_ext("fbw_core", "fbw_torch.cpp", lib_dir, lib_dir)
+    build_ext("fast_viterbi_core", "viterbi_torch.cpp", os.path.join(out_root, "fast_viterbi"), lib_dir)
 
 
 if __name__ == "__main__":

@@ -92,3 +92,20 @@ def test_static_entry_point_refuses_large_problems_on_the_host():
     with pytest.raises(cabi.FbwError) as e:
         cabi.run_static(256, 32 * 12001, 12001, 256, 30000, 256, 256, 32, 256, 1000, 32, 12001, 30000, 12000, 0, 256, 256, 0)
     assert e.value.code == cabi.ERR_STATIC_WORKSPACE
+
+
+def test_packaging_metadata():
+    """`pip install --no-build-isolation .` is driven by setup.py: its build step is the in-tree build routine
+    pointed at the build tree (the install itself compiles for minutes and is not run here)."""
+    import ast
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = open(os.path.join(root, "setup.py")).read()
+    tree = ast.parse(src)
+    names = {n.name for n in ast.walk(tree) if isinstance(n, (ast.ClassDef, ast.FunctionDef))}
+    assert {"BuildWithNative", "BinaryDistribution"} <= names
+    assert "build_all(os.path.join(self.build_lib" in src
+    assert os.path.exists(os.path.join(root, "pyproject.toml"))
+    from i6_native_ops_amd import build
+    import inspect
+    assert "out_root" in inspect.signature(build.build_all).parameters
