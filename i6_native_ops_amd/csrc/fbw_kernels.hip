@@ -2334,7 +2334,7 @@ struct Pipeline {
     bool attr_ready = false;  // kernel attributes set, device facts read
     bool ready = false;       // streams and events created
     hipStream_t sP = nullptr, sR = nullptr;
-    hipEvent_t start = nullptr, fork = nullptr, doneP = nullptr, doneR = nullptr;
+    hipEvent_t start = nullptr, fork = nullptr, gathered = nullptr, doneP = nullptr, doneR = nullptr;
     int n_cu = 256;
     int dense_regs = 0;       // vector registers per lane of fbw_recurse_dense<true>, as built
     // caller streams that were checked against the recursion stream: do kernels on the two run at
@@ -2389,7 +2389,7 @@ int pipeline_init(Pipeline& p) {
     // default priority on purpose
     HIP_TRY(hipStreamCreateWithFlags(&p.sP, hipStreamNonBlocking));
     HIP_TRY(hipStreamCreateWithFlags(&p.sR, hipStreamNonBlocking));
-    for (hipEvent_t* e : {&p.start, &p.fork, &p.doneP, &p.doneR})
+    for (hipEvent_t* e : {&p.start, &p.fork, &p.gathered, &p.doneP, &p.doneR})
         HIP_TRY(hipEventCreateWithFlags(e, hipEventDisableTiming));
     p.ready = true;
     return I6FBW_OK;
@@ -2673,14 +2673,14 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // precision (recurse_workgroup); it then takes two rounds.
     const bool dense = 2 * B > P.n_cu && T <= 4096;
     // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
-    // order of frames and sequences, rows are long enough for a span to cut only a few of them,
-    // and the stages overlap (for the small problems of the single-stream schedule the row writer
-    // is as good).
+    // order of frames and sequences, rows are long enough for a span to cut at most two of them,
+    // and the tensor is large (for small problems the row writer is as good).
     int flat_layout = -1;
     if (out_stride_b == (int64_t)F && out_stride_t == (int64_t)B * F) flat_layout = 0;
     else if (out_stride_t == (int64_t)F && out_stride_b == (int64_t)T * F) flat_layout = 1;
     const int writer = g_writer_mode.load();
-    bool flat = (writer > 0 || (writer < 0 && overlap)) && flat_layout >= 0 && F >= FLAT_MIN_F && l.wpfx_stride > 0;
+    bool flat = (writer > 0 || (writer < 0 && (overlap || (long long)T * B * F >= (1LL << 26)))) && flat_layout >= 0 &&
+                F >= FLAT_MIN_F && l.wpfx_stride > 0;
     FlatArgs fa;
     long long flat_grid = 0;
     if (flat) {
@@ -2751,18 +2751,8 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         HIP_TRY(hipStreamWaitEvent(sR, P.fork, 0));
         int rc = launch_recursion(); if (rc != I6FBW_OK) return rc;
     }
-    if (flat && overlap) {
-        // fbw_flat writes every row except those of sequences too large for its posterior jobs:
-        // these go row by row through fbw_combine on the second library stream, started once the
-        // preparation is done and all recursion workgroups are placed (its workgroups wait for the
-        // gather and the recursion while they hold wave slots); it has nothing to do for the usual
-        // batch.  The two kernels do not wait for each other.
-        if (early) HIP_TRY(hipEventRecord(P.fork, s));
-        HIP_TRY(hipStreamWaitEvent(sP, P.fork, 0));
-        hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, sP, sync, 2 * B);
-        { StageTimer tm(4, sP, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, sP, ca); }
-        HIP_TRY(hipGetLastError());
-    } else if (!flat) {
+    // (with the flat writer, the row writer for the sequences fbw_flat leaves out is started below, behind the gather)
+    if (!flat) {
         // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
         // leaves the memory system idle.
         StageTimer tm(4, sP, timed);
@@ -2794,6 +2784,19 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     HIP_TRY(hipGetLastError());
     { StageTimer tm(1, s, timed); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, s, ga); }
     HIP_TRY(hipGetLastError());
+    if (flat) {
+        // fbw_flat writes every row except those of sequences too large for its posterior jobs: these go
+        // row by row through fbw_combine on the second library stream, beside fbw_flat (the two kernels
+        // do not wait for each other).  It is started behind the gather like fbw_flat itself: its
+        // workgroups wait for the gather's strips while they hold registers and wave slots, so they
+        // must not be on the machine before the gather's own are (three of them fill a compute unit's
+        // register file).  It has nothing to do for the usual batch.
+        HIP_TRY(hipEventRecord(P.gathered, s));
+        HIP_TRY(hipStreamWaitEvent(sP, P.gathered, 0));
+        { StageTimer tm(4, sP, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, sP, ca); }
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipEventRecord(P.doneP, sP));
+    }
     // The dense write follows the gather on the same stream (its workgroups would only take wave
     // slots away from the gather before that: by then the two recursions are about to meet in the
     // middle of the sequences, where the dense write begins); each of its workgroups waits for the
