@@ -159,6 +159,18 @@ Layout make_layout(long long T, long long B, long long E, long long F = 1) {
 
 #ifdef I6_TRACE
 __device__ unsigned long long g_trace[4096];   // debug builds only: in-kernel timestamps
+__device__ inline unsigned long long trace_cu_key() {
+    const unsigned hw = __builtin_amdgcn_s_getreg(4 | (31 << 11)), xcc = __builtin_amdgcn_s_getreg(20 | (31 << 11));
+    return ((unsigned long long)(xcc & 15u) << 32) | ((hw >> 8) & 0xffu) | 0x100000000000ull;
+}
+__device__ inline void trace_corun(int slot) {
+    if (threadIdx.x == 0) {
+        const unsigned long long k = trace_cu_key();
+        int hit = 0, pair = 0;
+        for (int i = 0; i < 64; i++) { const unsigned long long r = g_trace[3000 + i]; hit |= r == k; pair |= (r ^ k) == 1; }
+        atomicAdd(&g_trace[slot], 1ull); if (hit) atomicAdd(&g_trace[slot + 1], 1ull); if (pair) atomicAdd(&g_trace[slot + 2], 1ull);
+    }
+}
 #endif
 
 // ---------------------------------------------------------------------------------------------
@@ -830,6 +842,9 @@ template <bool SYNC>
 __global__ __launch_bounds__(256) void fbw_gather(GatherArgs a) {
     int b, y;
     strip_index(a.B, &b, &y);
+#ifdef I6_TRACE
+    trace_corun(3110);
+#endif
     const SeqMeta m = a.meta[b];
     if (rec_class(m) <= 0) return;
     const int n = (m.L + TG - 1) / TG;
@@ -889,12 +904,18 @@ struct RecArgs {
 // pointers to those buffers must not be declared restrict.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Two ints behind the 32 floats of per-wave minima in a recursion workgroup's LDS: [0] whether the
+// workgroup runs at all (the wait for the preparation), [1] set by the loader wave when one of
+// its waits has run out.
+__device__ __forceinline__ int* rec_go_flag(float* wmin) { return (int*)(wmin + 32); }
+__device__ __forceinline__ int* rec_gave_up(float* wmin) { return (int*)(wmin + 32) + 1; }
+
 struct RecCursor {
     float* wp; long long wstep;      // workspace row written by the next step
     double* op; int ostep;           // its offset
     double c; bool pending;          // running offset, renormalisation requested by the last step
     int* progress; int nsteps;       // rows finished so far (SYNC), number of steps
-    const int* abort_flag;           // set by any wait of the call that has run out
+    const int* gave_up;              // LDS word the loader wave sets when a wait of its own has run out
 };
 
 // End of a step: the per-frame barrier and, every PUBLISH steps, the progress counter.  Stores
@@ -906,7 +927,10 @@ template <bool SYNC>
 __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
 #ifdef I6_TRACE
     if (threadIdx.x == 0 && (i % 50) == 0 && (blockIdx.x < 2 || blockIdx.x >= gridDim.x - 2))
+    {
         g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + i / 50] = wall_clock64();
+        g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + 32 + i / 50] = clock64();
+    }
 #endif
     static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
     const bool last = i + 1 == cur.nsteps;
@@ -915,16 +939,53 @@ __device__ __forceinline__ void step_end(const int i, RecCursor& cur) {
         if (last) wait_stores();
         else asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
     }
+#ifdef I6_TRACE
+    const bool tr_ = blockIdx.x == 0 && i >= 400 && i < 432 && (threadIdx.x & 63) == 0 && (threadIdx.x == 0 || threadIdx.x == 320);
+    if (tr_) g_trace[3200 + (threadIdx.x ? 64 : 0) + 2 * (i - 400)] = wall_clock64();
     lds_barrier();
-    // (not after a wait of this call has run out -- the loader wave's for a strip of the gather, for
-    // one: rows computed from then on may be built on scores that were not there yet, and whoever waits
-    // for them must run into its own limit and write NaN rather than use them)
-    if (pub && threadIdx.x == 0 && !load_agent(cur.abort_flag)) store_agent(cur.progress, last ? i + 2 : i + 2 - PUBLISH);
+    if (tr_) g_trace[3200 + (threadIdx.x ? 64 : 0) + 2 * (i - 400) + 1] = wall_clock64();
+#else
+    lds_barrier();
+#endif
+    // (not after the loader wave has given up waiting for a strip of the gather: rows computed from
+    // then on may be built on scores that were not there yet, and whoever waits for them must run into
+    // its own limit and write NaN rather than use them.  The loader says so in LDS: a flag in memory
+    // would cost this wave a round trip, and the other waves a wait at the next barrier, every time.)
+    if (pub && threadIdx.x == 0 && !*cur.gave_up) store_agent(cur.progress, last ? i + 2 : i + 2 - PUBLISH);
 }
 
 // One frame for the states tid + j*THREADS: predecessor values and staged emission scores from
 // LDS, log-sum-exp (base 2) in a fixed order, result to the other LDS buffer and the workspace.
 template <typename ST> __device__ __forceinline__ ST state_min(ST a, ST b) { return b < a ? b : a; }
+// minimum as one instruction; of a number and a NaN, the number
+__device__ __forceinline__ float num_min(float a, float b) { return __builtin_fminf(a, b); }
+__device__ __forceinline__ double num_min(double a, double b) { return __builtin_fmin(a, b); }
+
+// Value of a state after a frame, from the scores v[k] of its KT candidates (predecessor value +
+// edge weight + emission score): -log2 of the sum of the 2^-v[k], less the renormalisation `pend`.
+// Two candidates (left-to-right automata: stay or advance): min - log2(1 + 2^-|v0 - v1|), one exp2
+// instead of two and no comparison; inf - inf gives NaN, which the maximum with 0 replaces (the
+// result is then inf - 1 = inf, as it must be for a state none of whose predecessors is alive).
+template <int KT, typename ST, bool PEND>
+__device__ __forceinline__ ST state_value(const ST (&v)[KT], const float pend) {
+    if (KT == 2) {
+        const ST mn = num_min(v[0], v[1]);
+        const float d = __builtin_fmaxf(__builtin_fabsf((float)(v[0] - v[1])), 0.f);
+        const float l = __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(-d));
+        return (PEND ? mn - (ST)pend : mn) - (ST)l;
+    }
+    ST mn = v[0];
+#pragma unroll
+    for (int k = 1; k < KT; k++) mn = num_min(mn, v[k]);
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f((float)(mn - v[k]));
+    // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling.  With every
+    // candidate at +inf the differences are NaN and so is the result: the minimum with +inf, which
+    // returns the operand that is a number, turns it into the +inf it must be.
+    return num_min((PEND ? mn - (ST)pend : mn) - (ST)__builtin_amdgcn_logf(sum), (ST)INF_F);
+}
+
 
 // ST is the type of the state vector in LDS: float, or double for sequences whose alignment is so
 // constrained that the states carrying the posterior mass sit far from the frame minimum (their
@@ -951,17 +1012,9 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
     for (int j = 0; j < NJ; j++) {
         const int s = tid + j * THREADS;
         ST v[KT];
-        ST mn = (ST)INF_F;
 #pragma unroll
-        for (int k = 0; k < KT; k++) {
-            v[k] = *(const ST*)(stc + eo[j][k]) + (ST)(ew[j][k] + *(const float*)(amc + es[j][k]));
-            mn = state_min(mn, v[k]);
-        }
-        float sum = 0.f;
-#pragma unroll
-        for (int k = 0; k < KT; k++) sum += __builtin_amdgcn_exp2f((float)(mn - v[k]));
-        // sum is in [1, KT] whenever mn is finite: the raw log2 needs no range handling
-        const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
+        for (int k = 0; k < KT; k++) v[k] = *(const ST*)(stc + eo[j][k]) + (ST)(ew[j][k] + *(const float*)(amc + es[j][k]));
+        const ST r = state_value<KT, ST, true>(v, pend);
         stn[s] = r;
         if (s < SP) store_x<SYNC>(cur.wp + s, (float)r);
         rmin = fminf(rmin, (float)r);
@@ -976,22 +1029,97 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
     step_end<SYNC>(i, cur);
 }
 
+// One frame of a group of RENORM frames, its place in the group known at compile time: FIRST takes
+// up the renormalisation the previous group asked for (and writes the offsets of all rows of the
+// group, which share it: lanes 0..RENORM-1 of the first wave, one store each), LAST leaves the
+// wave's minimum for the next group.  The steps between them are nothing but the arithmetic, the
+// row store and the barrier (which the caller issues): the recursion is bound by the number of
+// instructions a SIMD has to issue per frame for the waves it holds.
+template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ, bool FIRST, bool LAST>
+__device__ __forceinline__ void recurse_step_in_group(const int SP, const char* stc, ST* stn, const char* amc, float* wmin,
+                                                      const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
+                                                      const float (&ew)[J][KT], RecCursor& cur) {
+    constexpr int NW = THREADS / 64;
+    const int tid = threadIdx.x;
+    float pend = 0.f;
+    if (FIRST) {
+        float mn = wmin[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) mn = fminf(mn, wmin[w]);
+        pend = mn == INF_F ? 0.f : mn;
+        cur.c += (double)pend;
+        if (tid < RENORM) store_x<SYNC>(cur.op + tid * cur.ostep, cur.c);
+        cur.op += RENORM * cur.ostep;
+    }
+    float rmin = INF_F;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        const int s = tid + j * THREADS;
+        ST v[KT];
+#pragma unroll
+        for (int k = 0; k < KT; k++) v[k] = *(const ST*)(stc + eo[j][k]) + (ST)(ew[j][k] + *(const float*)(amc + es[j][k]));
+        const ST r = state_value<KT, ST, FIRST>(v, pend);
+        stn[s] = r;
+        if (s < SP) store_x<SYNC>(cur.wp + s, (float)r);
+        if (LAST) rmin = fminf(rmin, (float)r);
+    }
+    cur.wp += cur.wstep;
+    if (LAST) {
+        rmin = wave_min_dpp(rmin);
+        if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
+    }
+}
+
 // all steps of a wave that has states in NJ of its J rounds
 template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ>
 __device__ __forceinline__ void recurse_time_loop(const int SP, ST* st0, ST* st1, const float* am0, const float* am1, float* wmin,
                                                   const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
                                                   const float (&ew)[J][KT], RecCursor& cur) {
-    for (int i = 0; i < cur.nsteps; i += 2) {
-        recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i, SP, (const char*)st0, st1, (const char*)am0, wmin, eo, es, ew, cur);
+    static_assert(RENORM == 8 && PUBLISH % RENORM == 0, "shape of a group of steps");
+    const char* c0 = (const char*)st0; const char* c1 = (const char*)st1;
+    const char* a0 = (const char*)am0; const char* a1 = (const char*)am1;
+    int i = 0;
+    // whole groups of RENORM steps, as long as the last step of the sequence is not among them
+    for (; i + RENORM < cur.nsteps; i += RENORM) {
+#ifdef I6_TRACE
+        if (threadIdx.x == 0 && (i % 48) == 0 && (blockIdx.x < 2 || blockIdx.x >= gridDim.x - 2)) {
+            g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + i / 48] = wall_clock64();
+            g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + 32 + i / 48] = clock64();
+        }
+#endif
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, true, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+        lds_barrier();
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+        lds_barrier();
+        for (int r = 0; r < (RENORM - 4) / 2; r++) {
+            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+            lds_barrier();
+            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+            lds_barrier();
+        }
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+        lds_barrier();
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, true>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+        // as step_end for the step i + RENORM - 1, which is never the last one
+        const bool pub = SYNC && ((i + RENORM) % PUBLISH) == 0;
+        static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
+        if (pub) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+        lds_barrier();
+        if (pub && threadIdx.x == 0 && !*cur.gave_up) store_agent(cur.progress, i + RENORM + 1 - PUBLISH);
+    }
+    cur.pending = i > 0;
+    // the rest, at most RENORM steps, the last one among them
+    for (; i < cur.nsteps; i += 2) {
+        recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i, SP, c0, st1, a0, wmin, eo, es, ew, cur);
         if (i + 1 < cur.nsteps)
-            recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i + 1, SP, (const char*)st1, st0, (const char*)am1, wmin, eo, es, ew, cur);
+            recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i + 1, SP, c1, st0, a1, wmin, eo, es, ew, cur);
     }
 }
 
 // common prologue of the compute waves: initial state vector, row 0 of the workspace, cursor
 template <bool SYNC, int THREADS, typename ST>
 __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m, const int b, const int dir, const int SCAP,
-                                             ST* st0, ST* st1, RecCursor& cur) {
+                                             ST* st0, ST* st1, float* wmin, RecCursor& cur) {
     const int tid = threadIdx.x;
     const int L = m.L, SP = m.SP, T = a.T;
     const long long soff = state_off(m.edge_begin, b);
@@ -1016,7 +1144,7 @@ __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m,
     cur.c = 0.0;
     cur.pending = false;
     cur.progress = a.sync + SYNC_HDR + 2 * b + dir;
-    cur.abort_flag = a.sync;
+    cur.gave_up = rec_gave_up(wmin);
     cur.nsteps = L - 1;
     if (SYNC) wait_stores();
     lds_barrier();
@@ -1054,7 +1182,7 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
     }
     if (tid < THREADS / 64) wmin[tid] = INF_F;
     RecCursor cur;
-    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
+    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, wmin, cur);
     // Rounds of this wave that hold a state at all (the cells of the others keep the +inf of the
     // start-up); the time loop is instantiated for that number, so that the LDS reads of all its
     // rounds are issued together.  Waves without a state leave: they would only compete with the
@@ -1087,7 +1215,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
     const uint2* ell = (dir ? a.ellB : a.ellA) + (size_t)KMAX * soff;
     const int K = dir ? m.Kout : m.Kin;
     RecCursor cur;
-    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, cur);
+    recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, wmin, cur);
     ST* stc = st0; ST* stn = st1;
     const float* amc = am0; const float* amn = am1;
     for (int i = 0; i < cur.nsteps; i++) {
@@ -1158,7 +1286,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
 // kernel has finished the strip a row belongs to.
 template <bool SYNC, int THREADS, int JL, int P>
 __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m, const int b, const int dir,
-                                             float* am0, float* am1) {
+                                             float* am0, float* am1, int* gave_up) {
     typedef unsigned long long u64;
     const int lane = threadIdx.x - THREADS;
     const int L = m.L, DP = m.DP, T = a.T;
@@ -1181,7 +1309,7 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
         const int f = dir ? L - 1 - ic : ic;
         if (SYNC && f / TG != strip_ok) {
             const int j = f / TG;
-            if (!(j == ahead_strip && ahead_val >= 1)) spin_until_ge(gflag + j, 1, abort_flag);
+            if (!(j == ahead_strip && ahead_val >= 1) && !spin_until_ge(gflag + j, 1, abort_flag)) *gave_up = 1;
             strip_ok = j;
             const int jn = dir ? j - 1 : j + 1;
             ahead_strip = -1;
@@ -1213,7 +1341,14 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
                 amn[lane + jl * 64] = g[q][jl];
                 g[q][jl] = load_x<SYNC>(nxt + cc(jl));
             }
+#ifdef I6_TRACE
+            { const int i_ = i0 + q; const bool tr_ = blockIdx.x == 0 && i_ >= 400 && i_ < 432 && lane == 0;
+              if (tr_) g_trace[3200 + 128 + 2 * (i_ - 400)] = wall_clock64();
+              lds_barrier();
+              if (tr_) g_trace[3200 + 128 + 2 * (i_ - 400) + 1] = wall_clock64(); }
+#else
             lds_barrier();
+#endif
             u64* t_ = amc; amc = amn; amn = t_;
         }
     }
@@ -1281,11 +1416,14 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     float (*amr)[D_MAX] = (float (*)[D_MAX])lds;
     float* stf = lds + 2 * D_MAX;                                        // state vectors, float or double
     float* wmin = stf + (DENSE ? 2 : 4) * (S_MAX + 16);
-    int* go_flag = (int*)(wmin + 32);      // wmin doubles as the 32-float scratch of the general path's reductions
+    int* go_flag = rec_go_flag(wmin);      // wmin doubles as the 32-float scratch of the general path's reductions
 
     // the recursion is the latency-critical kernel: its waves go first when they share a SIMD with
     // gather or combine waves
     __builtin_amdgcn_s_setprio(3);
+#ifdef I6_TRACE
+    if (threadIdx.x == 0 && blockIdx.x < 64) g_trace[3000 + blockIdx.x] = trace_cu_key();
+#endif
     if (SYNC) {
         // This kernel is started beside the preparation, so that its large workgroups are placed
         // while the machine is still empty: report the placement (see fbw_gate), wait until all
@@ -1293,6 +1431,7 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
         if (threadIdx.x == 0) {
             atomicAdd(&a.sync[1], 1);
             *go_flag = spin_until_ge(a.sync + 3, a.prep_wgs, a.sync) ? 1 : 0;
+            *rec_gave_up(wmin) = 0;
         }
         __syncthreads();
         if (!*go_flag) return;
@@ -1318,9 +1457,9 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     }
     if (cls <= 0) return;
     if (threadIdx.x >= T_) {
-        if (cls == 1) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1]);
-        else if (cls == 2) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1]);
-        else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1]);
+        if (cls == 1) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
+        else if (cls == 2) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
+        else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
         return;
     }
     // Double-precision state vectors where float would show in the posteriors.  State values are
@@ -1371,6 +1510,10 @@ __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS_F64];
     if (RESERVE) asm volatile("v_mov_b32 v167, 0" ::: "v167");
     recurse_workgroup<SYNC, false>(a, lds);
+#ifdef I6_TRACE
+    __syncthreads();
+    if (threadIdx.x == 0 && blockIdx.x < 64) g_trace[3000 + blockIdx.x] = 1;
+#endif
 }
 // The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS_F32 floats): with the
 // size known at compile time the compiler sees that at most two workgroups fit on a unit anyway
@@ -2242,6 +2385,7 @@ __global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs f
     }
 #ifdef I6_TRACE
     if (blk == 0 && threadIdx.x == 0) g_trace[2040] = wall_clock64();
+    trace_corun(3100);
 #endif
     if (i >= n) return;
     // middle: where the two recursions meet -- of the longest sequence (rows of all sequences of a
