@@ -2754,15 +2754,15 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     int* sync = (int*)(ws + l.sync);
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
     const int forced = static_call ? 0 : g_overlap_mode.load();
-    // By default only where it pays: a large dense tensor, and a batch whose recursion workgroups
-    // leave wave slots free on every compute unit (with two of them on each unit the gather crawls:
-    // T=200, B=256, F=5001 takes 0.49 ms overlapped against 0.40 ms stage after stage).
-    // Nor with few frames (there is little recursion to hide: up to 300 frames the stages in a row
-    // are as fast or up to 20 % faster at F = 12001) or, unless the sequences are long, with a handful
-    // of sequences (8 sequences of 1000 frames: 9 % slower overlapped; 8 of 4000 frames with large
-    // automata: 25 % faster).
+    // By default only where it pays (measured at F = 12001 unless said otherwise, ms per call stage
+    // after stage / overlapped): a large dense tensor; a batch whose recursion workgroups leave half of
+    // the compute units alone (T=400 B=100 F=5001: 0.33 / 0.36; T=200 B=256 F=5001: 0.34 / 0.43; with
+    // up to 64 sequences T=600 B=32: 0.37 / 0.33, T=1000 B=32: 0.62 / 0.52, T=2000 B=16 F=3000: 1.39 /
+    // 1.07); not with few frames (there is little recursion to hide: T=200 B=64 0.20 / 0.23, T=300 B=32
+    // 0.19 / 0.20) nor, unless the sequences are long, with a handful of sequences (T=1000 B=8: 0.36 /
+    // 0.34, T=4000 B=8 with large automata: 3.27 / 2.81).
     bool overlap = forced >= 0 ? forced != 0
-                               : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu && T >= 384 && (B >= 12 || T >= 2048));
+                               : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu / 2 && T >= 384 && (B >= 12 || T >= 1000));
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
     if (2 * B > (T <= 4096 ? 2 : 1) * P.n_cu) overlap = false;
