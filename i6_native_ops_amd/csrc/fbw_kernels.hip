@@ -279,6 +279,7 @@ struct PrepArgs {
     const int32_t* start_end; long long se_stride;
     const int32_t* seq_lens;
     int T, B, F, E, n_states;
+    int gate_need;      // > 0: a workgroup only ends when this many recursion workgroups are on the machine (see fbw_gate)
     int best_path;      // tables for the best-path search: weights unscaled, no source-ordered table
     int no_band;        // every (frame, slot) pair is gathered (debug dumps of the forward scores)
     int force_generic;  // F is too large for the emission bitmap: every sequence takes the general path
@@ -820,7 +821,12 @@ __global__ __launch_bounds__(NT) void fbw_prepare(PrepArgs a) {
     // The recursion kernel of the overlapped schedule is already on the machine and waits for this
     // count: write this workgroup's tables back from the L2 of its XCD before it is raised.
     __syncthreads();
-    if (threadIdx.x == 0) { __threadfence(); atomicAdd(&a.sync[3], 1); }
+    if (threadIdx.x == 0) {
+        __threadfence(); atomicAdd(&a.sync[3], 1);
+        // In place of the gate kernel, where the recursion was started ahead of this kernel: the gather
+        // follows in stream order, i.e. when the last of these workgroups has seen the recursion placed.
+        if (a.gate_need > 0) spin_until_ge(a.sync + 1, a.gate_need, a.sync);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2012,7 +2018,10 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
 // ---------------------------------------------------------------------------------------------
 constexpr int FLAT_W = 2048;                  // floats per span: two 16-byte stores per thread
 #ifndef I6_FLAT_AHEAD
-#define I6_FLAT_AHEAD 4
+#define I6_FLAT_AHEAD 6
+#endif
+#ifndef I6_FLAT_AHEAD_ALONE
+#define I6_FLAT_AHEAD_ALONE 4
 #endif
 #ifndef I6_FLAT_KMAX
 #define I6_FLAT_KMAX 8
@@ -2020,7 +2029,10 @@ constexpr int FLAT_W = 2048;                  // floats per span: two 16-byte st
 #ifndef I6_FLAT_OCC
 #define I6_FLAT_OCC 8
 #endif
-constexpr int FLAT_AHEAD = I6_FLAT_AHEAD;     // strips by which posterior jobs run ahead of the write jobs that need them
+// strips by which posterior jobs run ahead of the write jobs that need them: beside the recursion, whose
+// progress the posterior jobs wait for (headline 0.513 ms with 4, 0.508 with 6, 0.515 with 8), and with
+// everything ready when the kernel starts (config 4: dense write 0.193 ms with 4, 0.203 with 6)
+constexpr int FLAT_AHEAD = I6_FLAT_AHEAD, FLAT_AHEAD_ALONE = I6_FLAT_AHEAD_ALONE;
 constexpr int FLAT_KMAX = I6_FLAT_KMAX;       // spans per write job
 constexpr int FLAT_MIN_F = FLAT_W;            // a span then cuts at most two rows
 constexpr unsigned FLAT_SKIP = 0x7fc0deadu;   // image marker, a NaN no computation produces: element not written by this job
@@ -2030,6 +2042,7 @@ struct FlatArgs {
     int layout;            // 0: out is (T, B, F) contiguous, 1: (B, T, F) contiguous
     int nW;                // write jobs per group
     int K;                 // spans per write job
+    int ahead;             // strips by which posterior jobs are dispatched ahead of the write jobs that need them
     int shift;             // floats between the 128-byte line boundary below out and out
     int* cflag;            // per (sequence, strip): 1 compact posteriors written, 2 given up
     const int* wpfx; int wpfx_stride;
@@ -2375,13 +2388,13 @@ __global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs f
     constexpr int NQ = TC / FLAT_TCF;           // posterior jobs per strip of a sequence
     int i, b = -1, job = -1, qf = 0;            // job >= 0: write job number within its group; qf: which part of the strip
     const int blk = blockIdx.x;
-    if (blk < FLAT_AHEAD * B * NQ) { i = blk / (B * NQ); b = (blk / NQ) % B; qf = blk % NQ; }
+    if (blk < fa.ahead * B * NQ) { i = blk / (B * NQ); b = (blk / NQ) % B; qf = blk % NQ; }
     else {
-        const int x = blk - FLAT_AHEAD * B * NQ;
+        const int x = blk - fa.ahead * B * NQ;
         const int G = fa.nW + (fa.layout == 0 ? B : 1) * NQ;
         const int u = x / G, r = x % G;
-        if (fa.layout == 0) { i = u; if (r < fa.nW) job = r; else { b = (r - fa.nW) / NQ; qf = (r - fa.nW) % NQ; i += FLAT_AHEAD; } }
-        else { i = u / B; b = u % B; if (r < fa.nW) job = r; else { qf = r - fa.nW; i += FLAT_AHEAD; } }
+        if (fa.layout == 0) { i = u; if (r < fa.nW) job = r; else { b = (r - fa.nW) / NQ; qf = (r - fa.nW) % NQ; i += fa.ahead; } }
+        else { i = u / B; b = u % B; if (r < fa.nW) job = r; else { qf = r - fa.nW; i += fa.ahead; } }
     }
 #ifdef I6_TRACE
     if (blk == 0 && threadIdx.x == 0) g_trace[2040] = wall_clock64();
@@ -2835,7 +2848,8 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         fa.shift = row_misalign_host(out);
         fa.cflag = (int*)(ws + l.cflag); fa.wpfx = (const int*)(ws + l.wpfx); fa.wpfx_stride = l.wpfx_stride;
         fa.cp = ga.gtab;
-        flat_grid = (long long)FLAT_AHEAD * B * (TC / FLAT_TCF) + (flat_layout == 0 ? n : n * B) * (fa.nW + rows * (TC / FLAT_TCF));
+        fa.ahead = overlap ? FLAT_AHEAD : FLAT_AHEAD_ALONE;
+        flat_grid = (long long)fa.ahead * B * (TC / FLAT_TCF) + (flat_layout == 0 ? n : n * B) * (fa.nW + rows * (TC / FLAT_TCF));
         if (flat_grid > 0x7fffffffLL || (long long)TC * rows * F >= (1LL << 31) - FLAT_W) flat = false;
     }
     ca.direct_only = flat ? 1 : 0;
@@ -2852,6 +2866,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // least half of the compute units empty (the preparation's workgroups need most of a unit's
     // LDS and could otherwise find no room while the recursion waits for them), else behind it.
     const bool early = overlap && 2 * B <= P.n_cu / 2;
+    pa.gate_need = early ? 2 * B : 0;
     auto launch_recursion = [&]() -> int {
         { StageTimer tm(2, sR, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
           else if (early) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
@@ -2924,8 +2939,12 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // A running grid of small workgroups refills every wave slot it frees, so gather and dense
     // write (which also wait for recursion progress while they occupy LDS and wave slots) are
     // held back until every recursion workgroup is on the machine -- normally long since.
-    hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
-    HIP_TRY(hipGetLastError());
+    // (With the recursion started ahead of the preparation, the preparation's workgroups do that wait
+    // themselves at their end: one kernel less between preparation and gather.)
+    if (!early) {
+        hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
+        HIP_TRY(hipGetLastError());
+    }
     { StageTimer tm(1, s, timed); hipLaunchKernelGGL(fbw_gather<true>, g_grid, dim3(256), 0, s, ga); }
     HIP_TRY(hipGetLastError());
     if (flat) {
