@@ -2009,12 +2009,13 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
 // this kernel starts), so the job that is waited for is running or done: no wait can block the
 // kernel, whatever the occupancy.
 //
-// Measured on the headline tensor (1.54 GB): a bare writer of this shape reaches 6.9 TB/s with two
-// workgroups per compute unit and 5.9 with eight -- more stores on their way than the memory
-// system takes at a time cost bandwidth -- but a write job spends most of its life waiting for
-// what it reads (two dependent rounds of 2-3 us under this load), which takes all eight to hide;
-// this kernel writes the tensor in 0.265 ms when it has the machine to itself (5.8 TB/s, 0.30 ms
-// for fbw_combine + fbw_padfill) and in 0.26 ms of work beside the recursion.
+// Measured on the headline tensor (1.54 GB): bare writers with jobs of this shape (8 strided spans, built
+// in LDS, two 16-byte stores per thread) reach 5.6-5.9 TB/s whatever the occupancy, also as persistent
+// workers; 6.9 TB/s needs a fresh workgroup per single span at two per compute unit, i.e. jobs with
+// nothing to read.  This kernel writes the tensor in 0.265 ms when it has the machine to itself
+// (5.8 TB/s; 0.30 ms for fbw_combine + fbw_padfill) and spends the same beside the recursion.  Its time
+// does not change when the reads of the write jobs are taken out or when a workgroup waits for the
+// stores of each span before the next: it is bound by the memory system's rate for these writes.
 // ---------------------------------------------------------------------------------------------
 constexpr int FLAT_W = 2048;                  // floats per span: two 16-byte stores per thread
 #ifndef I6_FLAT_AHEAD
