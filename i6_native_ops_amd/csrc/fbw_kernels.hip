@@ -81,6 +81,18 @@ constexpr int REC_BLOCK = REC_THREADS + 64 * REC_LOADERS;
 // batches with more workgroups than compute units runs 448 compute threads beside the loader wave.
 constexpr int REC_THREADS_DENSE = 448;
 constexpr int REC_BLOCK_DENSE = REC_THREADS_DENSE + 64 * REC_LOADERS;
+// Batches of large automata (more than BIG_STATES states per sequence on average) run the instance with
+// fifteen compute waves: up to 960 states at one per thread, and half as many rounds beyond -- four
+// waves per SIMD with two states each overlap their LDS and arithmetic phases better than two with four
+// (8 sequences of 1350-1600 states over 2300-3700 frames: 2.83 -> 2.35 ms per call).  Small automata are
+// better off with fewer waves at the barrier (headline, 350-450 states: 0.507 ms against 0.533).
+constexpr int REC_THREADS_BIG = 960;
+constexpr int REC_BLOCK_BIG = REC_THREADS_BIG + 64 * REC_LOADERS;
+#ifndef I6_BIG_STATES
+#define I6_BIG_STATES 512
+#endif
+constexpr int BIG_STATES = I6_BIG_STATES;
+static_assert(REC_BLOCK_BIG <= 1024, "one workgroup");
 constexpr unsigned NO_STATE = 0xFFFFu;
 constexpr int SEQ_GENERIC = 1;        // value of SeqMeta::err / errA / errB that routes a sequence to the general path
 constexpr int SCAN_BLOCK = 1024;      // edges per workgroup of the sortedness scan
@@ -190,7 +202,7 @@ __device__ inline int rec_class(const SeqMeta& m, const int threads = REC_THREAD
     if (err < 0) return -1;
     if (m.L == 0 || m.n_edges == 0) return 0;
     if (err > 0) return -2;            // general path
-    if (m.SP <= threads && m.DP <= 512) return 1;
+    if (m.SP <= threads && m.DP <= (threads > 512 ? 1024 : 512)) return 1;     // (the loader wave of the large instance takes rows of 1024)
     if (m.SP <= 4 * threads && m.DP <= 2048) return 2;
     return 3;
 }
@@ -1199,7 +1211,7 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
     if (nj == 0) return;
     // (only in the instance for small batches: the one of which two workgroups share a compute unit
     // has no registers to spare for more loop bodies)
-    constexpr bool PER_ROUND = THREADS == REC_THREADS;
+    constexpr bool PER_ROUND = THREADS == REC_THREADS || THREADS == REC_THREADS_BIG;
     if (!PER_ROUND) recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
     else if (J == 1 || nj == 1) recurse_time_loop<SYNC, THREADS, J, KT, ST, 1>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
     else if (nj == 2) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 2 ? 2 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
@@ -1409,15 +1421,21 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
         if (K <= 2) recurse_compute<SYNC, T_, 4, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 4, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 4, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        // (degree 5-8 with at most two states per thread still fits the registers -- CTC automata, whose
+        // final states collect five edges: 603 states over 945 frames took 2.3 us per frame through the
+        // table-driven loop below -- but not under the register cap of the dense instance)
+        else if (T_ != REC_THREADS_DENSE && m.SP <= 2 * T_) recurse_compute<SYNC, T_, 2, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, 4 * T_);
     } else {
         recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, scap_big);
     }
 }
 
-template <bool SYNC, bool DENSE>
+// INST: 0 the instance for small batches, 1 the dense one (two workgroups per compute unit), 2 the one for large automata
+template <bool SYNC, int INST>
 __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) {
-    constexpr int T_ = DENSE ? REC_THREADS_DENSE : REC_THREADS;
+    constexpr bool DENSE = INST == 1;
+    constexpr int T_ = INST == 1 ? REC_THREADS_DENSE : (INST == 2 ? REC_THREADS_BIG : REC_THREADS);
     // LDS of a workgroup (16-byte aligned): the emission rows first
     float (*amr)[D_MAX] = (float (*)[D_MAX])lds;
     float* stf = lds + 2 * D_MAX;                                        // state vectors, float or double
@@ -1463,7 +1481,8 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     }
     if (cls <= 0) return;
     if (threadIdx.x >= T_) {
-        if (cls == 1) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
+        if (cls == 1 && INST == 2) recurse_load<SYNC, T_, 8, 4>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
+        else if (cls == 1) recurse_load<SYNC, T_, 4, 8>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
         else if (cls == 2) recurse_load<SYNC, T_, 16, 2>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
         else recurse_load<SYNC, T_, 32, 1>(a, m, b, dir, amr[0], amr[1], rec_gave_up(wmin));
         return;
@@ -1515,7 +1534,7 @@ template <bool SYNC, bool RESERVE = false>
 __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS_F64];
     if (RESERVE) asm volatile("v_mov_b32 v167, 0" ::: "v167");
-    recurse_workgroup<SYNC, false>(a, lds);
+    recurse_workgroup<SYNC, 0>(a, lds);
 #ifdef I6_TRACE
     __syncthreads();
     if (threadIdx.x == 0 && blockIdx.x < 64) g_trace[3000 + blockIdx.x] = 1;
@@ -1527,7 +1546,14 @@ __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
 template <bool SYNC>
 __global__ __launch_bounds__(REC_BLOCK_DENSE, 5) void fbw_recurse_dense(RecArgs a) {
     extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
-    recurse_workgroup<SYNC, true>(a, dyn_lds);
+    recurse_workgroup<SYNC, 1>(a, dyn_lds);
+}
+// Sixteen waves of at most 128 registers: the workgroup has its compute unit's register file to itself
+// without asking (see RESERVE above).
+template <bool SYNC>
+__global__ __launch_bounds__(REC_BLOCK_BIG) void fbw_recurse_big(RecArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds[REC_LDS_FLOATS_F64];
+    recurse_workgroup<SYNC, 2>(a, lds);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2830,6 +2856,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // the sequences can be longer than 4096 frames, which only the other instance runs in double
     // precision (recurse_workgroup); it then takes two rounds.
     const bool dense = 2 * B > P.n_cu && T <= 4096;
+    const bool big = !dense && (long long)n_states > (long long)BIG_STATES * B;
     // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
     // order of frames and sequences, rows are long enough for a span to cut at most two of them,
     // and the tensor is large (for small problems the row writer is as good).
@@ -2870,6 +2897,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     pa.gate_need = early ? 2 * B : 0;
     auto launch_recursion = [&]() -> int {
         { StageTimer tm(2, sR, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
+          else if (big) hipLaunchKernelGGL(fbw_recurse_big<true>, dim3(2 * B), dim3(REC_BLOCK_BIG), 0, sR, ra);
           else if (early) hipLaunchKernelGGL((fbw_recurse<true, true>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra);
           else hipLaunchKernelGGL((fbw_recurse<true, false>), dim3(2 * B), dim3(REC_BLOCK), 0, sR, ra); }
         HIP_TRY(hipGetLastError());
@@ -2926,6 +2954,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         { StageTimer tm(1, s, timed); hipLaunchKernelGGL(fbw_gather<false>, g_grid, dim3(256), 0, s, ga); }
         HIP_TRY(hipGetLastError());
         { StageTimer tm(2, s, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<false>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, s, ra);
+          else if (big) hipLaunchKernelGGL(fbw_recurse_big<false>, dim3(2 * B), dim3(REC_BLOCK_BIG), 0, s, ra);
           else hipLaunchKernelGGL(fbw_recurse<false>, dim3(2 * B), dim3(REC_BLOCK), 0, s, ra); }
         HIP_TRY(hipGetLastError());
         if (flat) {
