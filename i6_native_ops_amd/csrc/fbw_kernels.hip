@@ -1405,7 +1405,6 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
     const int K = dir ? m.Kout : m.Kin;
     // The loop body is specialised on the number of states per thread and of edge slots per state,
     // so that all LDS reads of a frame are issued back to back; unused slots read the +inf cell.
-    // (No six-edge specialisation for double: it is the rare case.)
     constexpr bool F32 = sizeof(ST) == 4;
     if (MANY && K > KMAX) {
         recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, scap_big);
@@ -1413,7 +1412,7 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
         if (K <= 2) recurse_compute<SYNC, T_, 1, 2, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 3) recurse_compute<SYNC, T_, 1, 3, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else if (K <= 4) recurse_compute<SYNC, T_, 1, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
-        else if (F32 && K <= 6) recurse_compute<SYNC, T_, 1, F32 ? 6 : KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (K <= 6) recurse_compute<SYNC, T_, 1, 6, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute<SYNC, T_, 1, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
     } else if (!MANY) {
         return;
@@ -1423,8 +1422,9 @@ __device__ __forceinline__ void recurse_dispatch(const RecArgs& a, const SeqMeta
         else if (K <= 4) recurse_compute<SYNC, T_, 4, 4, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         // (degree 5-8 with at most two states per thread still fits the registers -- CTC automata, whose
         // final states collect five edges: 603 states over 945 frames took 2.3 us per frame through the
-        // table-driven loop below -- but not under the register cap of the dense instance)
-        else if (T_ != REC_THREADS_DENSE && m.SP <= 2 * T_) recurse_compute<SYNC, T_, 2, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        // table-driven loop below)
+        else if (m.SP <= 2 * T_ && K <= 6) recurse_compute<SYNC, T_, 2, 6, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
+        else if (m.SP <= 2 * T_) recurse_compute<SYNC, T_, 2, KMAX, ST>(a, m, b, dir, st0, st1, am0, am1, wmin);
         else recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, 4 * T_);
     } else {
         recurse_compute_generic<SYNC, T_, ST>(a, m, b, dir, st0, st1, am0, am1, wmin, scap_big);
@@ -2792,6 +2792,13 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     char* ws = (char*)workspace;
     SeqMeta* meta = (SeqMeta*)(ws + l.meta);
     int* sync = (int*)(ws + l.sync);
+    // More recursion workgroups than compute units: the instance of which two fit on a unit -- unless
+    // the sequences can be longer than 4096 frames, which only the other instances run in double
+    // precision (recurse_workgroup), or the automata are too large for one state per thread there (with
+    // several states per thread and double vectors under its register cap it takes 1.5-1.8 us per frame
+    // where the other instances take 0.5: two rounds of those are faster).
+    const bool dense = 2 * B > P.n_cu && T <= 4096 && (long long)n_states <= (long long)REC_THREADS_DENSE * B;
+    const bool big = !dense && (long long)n_states > (long long)BIG_STATES * B;
     // Small problems run stage after stage on the caller's stream; large ones overlap the stages.
     const int forced = static_call ? 0 : g_overlap_mode.load();
     // By default only where it pays (measured at F = 12001 unless said otherwise, ms per call stage
@@ -2805,11 +2812,11 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
                                : ((long long)T * B * F >= (1LL << 26) && 2 * B <= P.n_cu / 2 && T >= 384 && (B >= 12 || T >= 1000));
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
-    if (2 * B > (T <= 4096 ? 2 : 1) * P.n_cu) overlap = false;
+    if (2 * B > (dense ? 2 : 1) * P.n_cu) overlap = false;
     // Two workgroups of the dense instance are four waves per SIMD: beyond 104 registers each they
     // leave no room for the gather's waves, which they wait for.  (The compiler is asked for 96; how
     // close it gets depends on its version.)
-    if (2 * B > P.n_cu && P.dense_regs > 104) overlap = false;
+    if (dense && P.dense_regs > 104) overlap = false;
     if (overlap) {
         // under stream capture: one stream, no in-memory waits between kernels, no synchronisation
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -2826,7 +2833,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
     pa.start_end = start_end; pa.se_stride = se_row_stride; pa.seq_lens = seq_lens;
-    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = (input_flags & I6FBW_IN_ALL_FRAMES) ? 1 : 0; pa.dense = (2 * B > P.n_cu && T <= 4096) ? 1 : 0; pa.force_generic = f_too_large ? 1 : 0;
+    pa.T = T; pa.B = B; pa.F = F; pa.E = E; pa.n_states = n_states; pa.best_path = 0; pa.no_band = (input_flags & I6FBW_IN_ALL_FRAMES) ? 1 : 0; pa.dense = dense ? 1 : 0; pa.force_generic = f_too_large ? 1 : 0;
     pa.meta = meta; pa.sync = sync; pa.sortflag = (int*)(ws + l.sortflag); pa.seqbegin = (int*)(ws + l.seqbegin); pa.eidx = (int*)(ws + l.eidx); pa.renum = (int2*)(ws + l.renum);
     pa.ellA = (uint2*)(ws + l.ellA); pa.ellB = (uint2*)(ws + l.ellB);
     pa.crec = (uint4*)(ws + l.crec); pa.cbegin = (int*)(ws + l.cbegin); pa.demis = (int*)(ws + l.demis); pa.tband = (int2*)(ws + l.tband);
@@ -2852,11 +2859,6 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     ca.tile_w = tiled ? COMB_TILE_W : 0;
     ca.direct_only = 0;
-    // More recursion workgroups than compute units: the instance of which two fit on a unit -- unless
-    // the sequences can be longer than 4096 frames, which only the other instance runs in double
-    // precision (recurse_workgroup); it then takes two rounds.
-    const bool dense = 2 * B > P.n_cu && T <= 4096;
-    const bool big = !dense && (long long)n_states > (long long)BIG_STATES * B;
     // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
     // order of frames and sequences, rows are long enough for a span to cut at most two of them,
     // and the tensor is large (for small problems the row writer is as good).

@@ -6,8 +6,9 @@ relative error <= 1e-5, posterior absolute error <= 1e-4 -- on random shapes of 
 families, under both schedules, and on shapes placed on either side of every one of those
 decisions: 1024 / 1025 frames, five states for three frames, 256 states with four frames each,
 and, for batches of more than 128 sequences (the recursion instance of which two workgroups share a
-compute unit), 383 / 384 frames, more than 1024 frames and more states than that instance has
-compute threads.  Every case is printed with its errors; the cases beyond the bar fail the test.
+compute unit, used while the automata are small on average), 383 / 384 frames, more than 1024 frames and more
+states than that instance has compute threads; batches of large automata (more than 512 states on
+average) run a third instance with fifteen compute waves.  Every case is printed with its errors; the cases beyond the bar fail the test.
 """
 import numpy as np
 import pytest
@@ -113,6 +114,28 @@ def test_large_batch_with_one_sequence_beyond_the_double_capacity_of_its_instanc
     failures = []
     for overlap in (0, 1):
         check(oracle, W, overlap, f"129 small + 1 of 2101 states, overlap={overlap}", failures)
+    assert not failures, failures
+
+
+def test_large_batch_with_a_few_sequences_of_several_states_per_thread(oracle):
+    """A batch of more than 128 sequences runs the recursion instance of which two workgroups share a compute
+    unit only while its automata are small on average; this one is (120 small CTC automata), and its ten
+    chain automata of 601 states over up to 1100 frames take that instance's path for several states per thread,
+    in double."""
+    from tests.test_flat_writer_gpu import merge
+    T = 1100
+    small = make_workload("ctc", seed=81, T=T, B=120, F=97, n_labels=(20, 40))
+    mid = make_workload("cart", seed=82, T=T, B=10, F=97, n_labels=(200, 200))
+    mid.seq_lens[:] = np.resize(np.asarray([T, T - 1, 700, 1024, 1025], dtype=np.int32), 10)
+    am, edges, weights, se, lens, n_states = merge([small, mid])
+
+    class W:
+        pass
+    W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states = am, edges, weights, se, lens, n_states
+    assert n_states <= 448 * 130
+    failures = []
+    for overlap in (0, 1):
+        check(oracle, W, overlap, f"120 small + 10 of 601 states, overlap={overlap}", failures)
     assert not failures, failures
 
 
