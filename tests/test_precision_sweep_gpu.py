@@ -139,6 +139,28 @@ def test_large_batch_with_a_few_sequences_of_several_states_per_thread(oracle):
     assert not failures, failures
 
 
+def test_one_large_automaton_of_higher_degree_among_small_ones(oracle):
+    """Six small CTC automata and one of 603 states: the batch runs the instance with eight compute waves
+    (small automata on average), and the large one, whose final state collects five edges, keeps two states per
+    thread with its edges in registers; 1203 states take the table-driven loop."""
+    from tests.test_flat_writer_gpu import merge
+    failures = []
+    for n in (300, 600):
+        T = 2 * n + 200
+        small = make_workload("ctc", seed=91, T=T, B=6, F=211, n_labels=(30, 50))
+        large = make_workload("ctc", seed=92, T=T, B=1, F=211, n_labels=(n, n))
+        large.seq_lens[:] = T - 5
+        am, edges, weights, se, lens, n_states = merge([small, large])
+
+        class W:
+            pass
+        W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states = am, edges, weights, se, lens, n_states
+        assert n_states <= 512 * 7
+        for overlap in (0, 1):
+            check(oracle, W, overlap, f"6 small + 1 CTC automaton of {2 * n + 3} states, overlap={overlap}", failures)
+    assert not failures, failures
+
+
 def test_random_shapes(oracle):
     """160 random cases: family, size, tightness of the alignment, edge order, batch size, schedule."""
     rng = np.random.default_rng(20241)

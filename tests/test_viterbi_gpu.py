@@ -104,11 +104,15 @@ def test_workloads(oracle, name, shuffle):
     assert_identical(got, want)
 
 
-@pytest.mark.parametrize("kind", ["cart_small", "large_states", "large_emissions", "huge_states"])
+@pytest.mark.parametrize("kind", ["cart_small", "large_states", "large_emissions", "huge_states", "ctc_two_per_thread", "ctc_table"])
 def test_size_classes(oracle, kind):
     """Chains that take the one-state-per-thread path, the four-states-per-thread path (more than 512
-    states or distinct emissions) and the table-in-memory path (more than 2048 states)."""
-    if kind == "cart_small":
+    states or distinct emissions) and the table-in-memory path (more than 2048 states); CTC automata
+    (five edges into the final state) of 603 states -- two per thread, edges in registers -- and of 1203."""
+    if kind.startswith("ctc"):
+        n = 300 if kind == "ctc_two_per_thread" else 600
+        wl = make_workload("ctc", T=2 * n + 150, B=2, F=700, n_labels=(n, n))
+    elif kind == "cart_small":
         wl = make_workload("cart", T=300, B=4, F=12001, n_labels=(60, 90))
     elif kind == "large_states":
         wl = make_workload("cart", T=900, B=2, F=300, n_labels=(250, 280))
