@@ -1582,8 +1582,11 @@ typedef float float4a __attribute__((ext_vector_type(4)));
 // ones and for those on the general path.  Sequences with a reported problem or without edges have
 // constant rows, which the write jobs of fbw_flat produce by themselves.
 constexpr int COMB_FAST_EDGES = 1024, COMB_FAST_SLOTS = 512;
+// (fbw_flat: up to COMB_FAST_* everything of a thread stays in registers over the frames of a job; up to
+// FLAT_* the edges are taken in pieces of COMB_FAST_EDGES per frame, their scores parked in the staging area)
+constexpr int FLAT_EDGES = 2048, FLAT_SLOTS = 1024;
 __device__ __forceinline__ bool flat_fast(const SeqMeta& m) {
-    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= COMB_FAST_EDGES && m.D <= COMB_FAST_SLOTS;
+    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= FLAT_EDGES && m.D <= FLAT_SLOTS;
 }
 __device__ __forceinline__ bool flat_direct(const SeqMeta& m) {
     return seq_error(m) >= 0 && m.n_edges > 0 && m.L > 0 && !flat_fast(m);
@@ -2136,8 +2139,82 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
     const float* gbase = a.gtab + (size_t)T * goff;
     float* cpbase = fa.cp + (size_t)T * goff;
 
+    constexpr int JE = COMB_FAST_EDGES / COMB_THREADS;
+    if (nE > COMB_FAST_EDGES || D > COMB_FAST_SLOTS) {
+        // Larger sequences: the edges of a frame in pieces of COMB_FAST_EDGES (records re-read from the
+        // cache per frame), raw scores parked in the staging area until the frame minimum is known.
+        constexpr int JSL = FLAT_SLOTS / COMB_THREADS;
+        static_assert(FLAT_W >= FLAT_EDGES, "the staging area holds the scores of all edges");
+        unsigned crl[JSL];
+#pragma unroll
+        for (int js = 0; js < JSL; js++) {
+            const int d = tid + js * COMB_THREADS;
+            crl[js] = d < D ? (unsigned)cb[d] | ((unsigned)cb[d + 1] << 16) : 0u;
+        }
+        for (int t = t0; t < tv; t++) {
+            const float* arow = abase + (size_t)t * SP;
+            const float* brow = bbase + (size_t)t * SP;
+            const float* grow = gbase + (size_t)t * DP;
+            double offs = 0.0;
+            if (tid == 0) offs = load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t);
+            float lmin = INF_F;
+            for (int c0 = 0; c0 < nE; c0 += COMB_FAST_EDGES) {
+                uint4 r[JE];
+                float va[JE], vb[JE], vg[JE];
+#pragma unroll
+                for (int j = 0; j < JE; j++) {
+                    const int i = c0 + tid + j * COMB_THREADS;
+                    r[j] = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+                    if (i < nE) r[j] = crec[i];
+                }
+#pragma unroll
+                for (int j = 0; j < JE; j++) {
+                    va[j] = load_x<SYNC>(arow + (r[j].x & 0xFFFFu)); vb[j] = load_x<SYNC>(brow + (r[j].x >> 16)); vg[j] = load_x<SYNC>(grow + r[j].z);
+                }
+#pragma unroll
+                for (int j = 0; j < JE; j++) {
+                    const int i = c0 + tid + j * COMB_THREADS;
+                    const float x = (va[j] + __uint_as_float(r[j].y)) + (vg[j] + vb[j]);     // same order as below
+                    if (i < nE) xs[i] = x;
+                    lmin = fminf(lmin, x);
+                }
+            }
+            const float mn = block_min256(lmin, redmin);
+            for (int i = tid; i < nE; i += COMB_THREADS) xs[i] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - xs[i]);    // (each thread its own)
+            __syncthreads();
+            float sd[JSL];
+            float lsum = 0.f;
+#pragma unroll
+            for (int js = 0; js < JSL; js++) {
+                sd[js] = slot_sum(xs, (int)(crl[js] & 0xFFFFu), (int)(crl[js] >> 16));
+                lsum += sd[js];
+            }
+            const float tot = block_sum256(lsum, redsum);
+            const bool dead = mn == INF_F;
+            const float logtot = __builtin_amdgcn_logf(tot);
+            if (tid == 0)
+                a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)(((double)(mn - logtot) + offs) * (double)LN2);
+            const float inv = dead ? 0.f : psign / tot;
+            float* cprow = cpbase + (size_t)t * DP;
+#pragma unroll
+            for (int js = 0; js < JSL; js++) {
+                const int d = tid + js * COMB_THREADS;
+                if (d < D) {
+                    float v;
+                    if (prob) v = sd[js] * inv;
+                    else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+                    store_agent(cprow + d, v);
+                }
+            }
+            __syncthreads();        // the staging area is written again for the next frame
+        }
+        wait_stores();
+        __syncthreads();
+        if (tid == 0) store_agent(flag, 1);
+        return;
+    }
     // this thread's edges and slots stay in registers for the whole strip
-    constexpr int JE = COMB_FAST_EDGES / COMB_THREADS, JS = COMB_FAST_SLOTS / COMB_THREADS;
+    constexpr int JS = COMB_FAST_SLOTS / COMB_THREADS;
     unsigned eft[JE], esl[JE];
     float ew[JE];
 #pragma unroll
@@ -2294,22 +2371,25 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
 #endif
     // Slots of the pieces -> registers.  Piece i belongs to the LP lanes from i * LP on; each of them
     // takes every LP-th slot of the piece, up to NSP of them: position within the span (-1: none)
-    // and value.  A piece with more slots than that (rare: more than a thirty-second of its emissions
-    // in use) is completed in the span loop below.
+    // and value.  With LP = 16 lanes per piece the 16 pieces of the job are fetched in one round, which
+    // covers pieces of up to 128 slots; a job with fuller pieces (sequences that use more than a
+    // sixteenth of the emissions) takes its spans four or two at a time with 32 or 64 lanes per piece,
+    // and what is still left of a piece then is fetched while its span is built.
     constexpr int LP = COMB_THREADS / (2 * FLAT_KMAX), NSP = 8;
     static_assert(LP * 2 * FLAT_KMAX == COMB_THREADS && LP >= 1, "lanes per piece");
-    const int mine = tid / LP, ln = tid % LP;          // my piece, my lane within it
     int q[NSP];
     float v[NSP];
-    const bool have = mine < 2 * nspans && s_kind[mine] == 1;
-    {
+    // pieces 2 * k0 ... of the job, lp lanes each
+    auto fetch_pieces = [&](const int k0, const int lp) {
+        const int mine = 2 * k0 + tid / lp, ln = tid % lp;          // my piece, my lane within it
+        const bool have = mine < 2 * nspans && s_kind[mine] == 1;
         // (all loads are issued before the first result is used: index and value do not depend on each other)
         const int s0 = have ? s_lo[mine] : 0, s1 = have ? s_hi[mine] : 0;
         const int* de = a.demis + (have ? s_de[mine] : 0);
         const float* cprow = fa.cp + (have ? s_cp[mine] : 0);
 #pragma unroll
         for (int n = 0; n < NSP; n++) {
-            const int sl = s0 + ln + n * LP;
+            const int sl = s0 + ln + n * lp;
             q[n] = -1; v[n] = 0.f;
             if (sl < s1) { q[n] = de[sl]; v[n] = load_agent(cprow + sl); }
         }
@@ -2321,16 +2401,10 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
                 q[n] = (pos >= p0 && pos < p1) ? pos : -1;
             }
         }
-    }
-    bool crowded = false;
-    for (int i = 0; i < 2 * nspans; i++) crowded = crowded || (s_kind[i] == 1 && s_hi[i] - s_lo[i] > LP * NSP);
+    };
     float* dst0 = (a.out - fa.shift) + first;
-#ifdef I6_TRACE
-    if (traced) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); tr[2] = wall_clock64(); }
-#endif
-#pragma unroll
-    for (int k = 0; k < FLAT_KMAX; k++) {
-        if (k >= nspans) break;
+    // span k of the job: mine = whether my registers hold values of it, held = slots per piece that the registers cover
+    auto emit_span = [&](const int k, const bool mine, const int held, const bool check_rest) {
         const long long span0 = first + (long long)(job + k * fa.nW) * FLAT_W;
         const int ka = s_kind[2 * k], kb = s_kind[2 * k + 1];
         // Spans that need care: cut by an end of the group, or holding a piece that is constant (NaN) or
@@ -2350,16 +2424,16 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
             for (int i = (int)max(0LL, g1 - span0) + tid; i < FLAT_W; i += COMB_THREADS) image[i] = __uint_as_float(FLAT_SKIP);
         }
         // the image holds holes everywhere else (see below); now my values of this span
-        if ((mine >> 1) == k) {
+        if (mine) {
 #pragma unroll
             for (int n = 0; n < NSP; n++)
                 if (q[n] >= 0) image[q[n]] = v[n];
         }
-        if (crowded) {
+        if (check_rest) {
             for (int w = 0; w < 2; w++) {
                 const int i = 2 * k + w;
                 if (s_kind[i] != 1) continue;
-                for (int sl = s_lo[i] + LP * NSP + tid; sl < s_hi[i]; sl += COMB_THREADS) {
+                for (int sl = s_lo[i] + held + tid; sl < s_hi[i]; sl += COMB_THREADS) {
                     const int pos = s_at[i] + a.demis[s_de[i] + sl];
                     if (pos >= s_p0[i] && pos < s_p1[i]) image[pos] = load_agent(fa.cp + s_cp[i] + sl);
                 }
@@ -2392,9 +2466,30 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
         img4[tid] = hole4;
         img4[tid + COMB_THREADS] = hole4;
         lds_barrier();
+    };
+    int fullest = 0;
+    for (int i = 0; i < 2 * nspans; i++) if (s_kind[i] == 1) fullest = max(fullest, s_hi[i] - s_lo[i]);
+    if (fullest <= LP * NSP) {
+        fetch_pieces(0, LP);
 #ifdef I6_TRACE
-        if (traced) tr[3 + k] = wall_clock64();
+        if (traced) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); tr[2] = wall_clock64(); }
 #endif
+#pragma unroll
+        for (int k = 0; k < FLAT_KMAX; k++) {
+            if (k >= nspans) break;
+            emit_span(k, ((tid / LP) >> 1) == k, LP * NSP, false);
+#ifdef I6_TRACE
+            if (traced) tr[3 + k] = wall_clock64();
+#endif
+        }
+    } else {
+        const int lp = fullest <= 2 * LP * NSP ? 2 * LP : 4 * LP;
+        const int per_round = COMB_THREADS / (2 * lp);          // spans whose pieces one round of registers holds
+        for (int k0 = 0; k0 < nspans; k0 += per_round) {
+            fetch_pieces(k0, lp);
+            for (int k = k0; k < min(nspans, k0 + per_round); k++)
+                emit_span(k, ((tid / lp) >> 1) == k - k0, lp * NSP, fullest > lp * NSP);
+        }
     }
 #ifdef I6_TRACE
     if (traced) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); tr[12] = wall_clock64(); }

@@ -4,7 +4,7 @@ writer and the oracle, through the C ABI.
 Both writers run the same per-frame arithmetic in the same order, so their outputs must be
 identical bit for bit, in every output mode, in both contiguous layouts, at any alignment of the
 output tensor, and for batches that mix ordinary sequences with ones the flat kernel leaves to
-the row kernel (too large for its posterior jobs), ones with a reported problem (NaN rows), ones
+the row kernel (too large for its posterior jobs), ones whose edges those jobs take in pieces, ones with a reported problem (NaN rows), ones
 without edges and ones without frames.
 """
 import numpy as np
@@ -78,12 +78,15 @@ def run(args, writer, out_mode, layout, misalign, overlap=1):
 
 
 def mixed_batch(T, F, seed):
-    """five ordinary sequences, one too large for the flat kernel's posterior jobs, and degenerate ones"""
+    """five ordinary sequences, one whose edges the flat kernel's posterior jobs take in two pieces, one too
+    large for them (left to the row kernel), and degenerate ones"""
     small = make_workload("cart", seed=seed, T=T, B=8, F=F, n_labels=(4, max(5, T // 12)))
     large = make_workload("cart", seed=seed + 1, T=T, B=1, F=F, n_labels=(180, 180))      # 1080 edges
     large.seq_lens[:] = T
+    huge = make_workload("cart", seed=seed + 3, T=T, B=1, F=F, n_labels=(350, 350))       # 2100 edges
+    huge.seq_lens[:] = T
     ctc = make_workload("ctc", seed=seed + 2, T=T, B=2, F=F, n_labels=(3, max(4, T // 8)))
-    args = list(merge([small, large, ctc]))
+    args = list(merge([small, large, ctc, huge]))
     lens = args[4]
     lens[1] = 0                # no frames at all
     lens[2] = T + 5            # out of range: treated like 0 (fbw_op.cu:61-69 never seeds beta)
@@ -105,6 +108,8 @@ def mixed_batch(T, F, seed):
     (33, 12001, 1, 0, 2),
     (560, 300, 0, 4, 1),       # long enough for the large sequence (540 states) to carry mass
     (560, 200, 1, 0, 0),
+    (600, 2048, 0, 0, 1),      # the same with rows long enough for the flat writer
+    (1100, 2050, 1, 6, 0),     # and for the one of 1051 states that is left to the row kernel
 ])
 def test_flat_writer_equals_row_writer_and_oracle(oracle, T, F, layout, misalign, out_mode):
     from i6_native_ops_amd import cabi
