@@ -2144,41 +2144,61 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
         // Larger sequences: the edges of a frame in pieces of COMB_FAST_EDGES (records re-read from the
         // cache per frame), raw scores parked in the staging area until the frame minimum is known.
         constexpr int JSL = FLAT_SLOTS / COMB_THREADS;
-        static_assert(FLAT_W >= FLAT_EDGES, "the staging area holds the scores of all edges");
+        float* xs_all = xs;       // scores of all edges, frame by frame
         unsigned crl[JSL];
 #pragma unroll
         for (int js = 0; js < JSL; js++) {
             const int d = tid + js * COMB_THREADS;
             crl[js] = d < D ? (unsigned)cb[d] | ((unsigned)cb[d + 1] << 16) : 0u;
         }
-        for (int t = t0; t < tv; t++) {
-            const float* arow = abase + (size_t)t * SP;
-            const float* brow = bbase + (size_t)t * SP;
-            const float* grow = gbase + (size_t)t * DP;
-            double offs = 0.0;
-            if (tid == 0) offs = load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t);
-            float lmin = INF_F;
-            for (int c0 = 0; c0 < nE; c0 += COMB_FAST_EDGES) {
-                uint4 r[JE];
-                float va[JE], vb[JE], vg[JE];
+        // (a piece of the edge records serves all frames of the job: one round trip for the records, one for
+        // the operands of all frames, per piece)
+        const int nf = tv - t0;
+        float lmins[FLAT_TCF];
+        double voffs[FLAT_TCF];
+#pragma unroll
+        for (int f = 0; f < FLAT_TCF; f++) {
+            lmins[f] = INF_F; voffs[f] = 0.0;
+            if (tid == 0 && f < nf) voffs[f] = load_x<SYNC>(offA + t0 + f) + load_x<SYNC>(offB + t0 + f);
+        }
+        for (int c0 = 0; c0 < nE; c0 += COMB_FAST_EDGES) {
+            uint4 r[JE];
+            float va[FLAT_TCF][JE], vb[FLAT_TCF][JE], vg[FLAT_TCF][JE];
+#pragma unroll
+            for (int j = 0; j < JE; j++) {
+                const int i = c0 + tid + j * COMB_THREADS;
+                r[j] = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+                if (i < nE) r[j] = crec[i];
+            }
+#pragma unroll
+            for (int f = 0; f < FLAT_TCF; f++) {
+                const int t = min(t0 + f, tv - 1);
+                const float* arow = abase + (size_t)t * SP;
+                const float* brow = bbase + (size_t)t * SP;
+                const float* grow = gbase + (size_t)t * DP;
 #pragma unroll
                 for (int j = 0; j < JE; j++) {
-                    const int i = c0 + tid + j * COMB_THREADS;
-                    r[j] = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
-                    if (i < nE) r[j] = crec[i];
-                }
-#pragma unroll
-                for (int j = 0; j < JE; j++) {
-                    va[j] = load_x<SYNC>(arow + (r[j].x & 0xFFFFu)); vb[j] = load_x<SYNC>(brow + (r[j].x >> 16)); vg[j] = load_x<SYNC>(grow + r[j].z);
-                }
-#pragma unroll
-                for (int j = 0; j < JE; j++) {
-                    const int i = c0 + tid + j * COMB_THREADS;
-                    const float x = (va[j] + __uint_as_float(r[j].y)) + (vg[j] + vb[j]);     // same order as below
-                    if (i < nE) xs[i] = x;
-                    lmin = fminf(lmin, x);
+                    va[f][j] = load_x<SYNC>(arow + (r[j].x & 0xFFFFu)); vb[f][j] = load_x<SYNC>(brow + (r[j].x >> 16)); vg[f][j] = load_x<SYNC>(grow + r[j].z);
                 }
             }
+#pragma unroll
+            for (int f = 0; f < FLAT_TCF; f++) {
+#pragma unroll
+                for (int j = 0; j < JE; j++) {
+                    const int i = c0 + tid + j * COMB_THREADS;
+                    const float x = (va[f][j] + __uint_as_float(r[j].y)) + (vg[f][j] + vb[f][j]);     // same order as below
+                    if (i < nE) xs_all[f * FLAT_EDGES + i] = x;
+                    lmins[f] = fminf(lmins[f], x);
+                }
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < FLAT_TCF; f++) {
+            if (f >= nf) break;
+            const int t = t0 + f;
+            float* xs = xs_all + f * FLAT_EDGES;
+            const float lmin = lmins[f];
+            const double offs = voffs[f];
             const float mn = block_min256(lmin, redmin);
             for (int i = tid; i < nE; i += COMB_THREADS) xs[i] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - xs[i]);    // (each thread its own)
             __syncthreads();
@@ -2206,7 +2226,6 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
                     store_agent(cprow + d, v);
                 }
             }
-            __syncthreads();        // the staging area is written again for the next frame
         }
         wait_stores();
         __syncthreads();
@@ -2498,7 +2517,9 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
 
 template <bool SYNC>
 __global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs fa) {
-    __shared__ float4a img4[FLAT_W / 4];        // image of a write job; staging area of a posterior job
+    // image of a write job; staging area of a posterior job (the scores of the edges of its frames)
+    __shared__ float4a img4[FLAT_TCF * FLAT_EDGES / 4];
+    static_assert(FLAT_TCF * FLAT_EDGES >= FLAT_W, "the image fits");
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
     __shared__ int s_kind[12 * FLAT_KMAX];
