@@ -3012,7 +3012,12 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // least half of the compute units empty (the preparation's workgroups need most of a unit's
     // LDS and could otherwise find no room while the recursion waits for them), else behind it.
     const bool early = overlap && 2 * B <= P.n_cu / 2;
-    pa.gate_need = early ? 2 * B : 0;
+    // The preparation's workgroups can do the gate's wait themselves (one kernel less in front of the gather)
+    // where they cannot be in the recursion's way: a preparation workgroup and a recursion workgroup do not
+    // share a compute unit, the order in which the two kernels are placed is not ours, and a preparation
+    // workgroup that waits keeps its unit -- so only if both grids fit with a unit per workgroup.
+    const bool gate_in_prepare = early && 5 * B <= P.n_cu;
+    pa.gate_need = gate_in_prepare ? 2 * B : 0;
     auto launch_recursion = [&]() -> int {
         { StageTimer tm(2, sR, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);
           else if (big) hipLaunchKernelGGL(fbw_recurse_big<true>, dim3(2 * B), dim3(REC_BLOCK_BIG), 0, sR, ra);
@@ -3087,9 +3092,8 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // A running grid of small workgroups refills every wave slot it frees, so gather and dense
     // write (which also wait for recursion progress while they occupy LDS and wave slots) are
     // held back until every recursion workgroup is on the machine -- normally long since.
-    // (With the recursion started ahead of the preparation, the preparation's workgroups do that wait
-    // themselves at their end: one kernel less between preparation and gather.)
-    if (!early) {
+    // (Or by the preparation's workgroups at their end, see gate_in_prepare.)
+    if (!gate_in_prepare) {
         hipLaunchKernelGGL(fbw_gate, dim3(1), dim3(64), 0, s, sync, 2 * B);
         HIP_TRY(hipGetLastError());
     }
