@@ -89,3 +89,112 @@ def test_full_size_best_path(oracle):
         L = int(W.seq_lens[b])
         em = float((-W.am_scores[np.arange(L), b, a[:L, b]]).astype(np.float64).sum())
         assert float(scores[b]) <= em + 1e-3
+
+
+def _check_sequences_against_oracle(oracle, W, am, post, loss, which):
+    """The oracle on a few sequences of a batch whose scores live on the device only."""
+    which = np.asarray(which)
+    am_sub = np.ascontiguousarray(am[:, torch.from_numpy(which).to(am.device), :].cpu().numpy())
+    keep = np.isin(W.edges[3], which)
+    edges = W.edges[:, keep].copy()
+    edges[3] = np.searchsorted(which, edges[3])
+    want_out, want_loss = oracle.fbw_oracle(am_sub, edges, W.weights[keep].copy(), W.start_end_states[:, which].copy(),
+                                            W.seq_lens[which].copy(), W.n_states, threads=len(which))
+    for k, b in enumerate(which):
+        np.testing.assert_allclose(loss[:, b].cpu().numpy(), want_loss[:, k], rtol=1e-5, atol=1e-6)
+        ref = np.exp(-want_out[:, k].astype(np.float64))
+        worst = float(np.abs(post[:, b].cpu().numpy() - ref).max())
+        assert worst <= 1e-4, (int(b), worst)
+
+
+@pytest.mark.parametrize("writer", [-1, 0], ids=["library_choice", "row_writer"])
+@pytest.mark.parametrize("layout", ["tbf", "btf"])
+def test_more_than_2_to_31_elements(oracle, writer, layout):
+    """T*B*F = 2.3e9: element offsets into scores and result do not fit 32 bits from frame 932 on
+    (time-major) or from sequence 179 on (batch-major).  Scores are drawn on the device; properties over the whole
+    result, the oracle on three sequences (first, middle, last)."""
+    B = 192
+    W = make_workload("cart", B=B, with_am=False)
+    T, F = W.T, W.F
+    assert T * B * F > 2 ** 31
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(77)
+    am = torch.empty((T, B, F), dtype=torch.float32, device=dev)
+    for t0 in range(0, T, 50):
+        x = torch.randn((min(50, T - t0), B, F), generator=gen, device=dev) * 3.0
+        am[t0:t0 + 50] = -torch.log_softmax(x.double(), -1).float()
+    del x
+    d = dict(edges=torch.from_numpy(W.edges).to(dev), w=torch.from_numpy(W.weights).to(dev),
+             se=torch.from_numpy(W.start_end_states).to(dev), lens=torch.from_numpy(W.seq_lens).to(dev))
+    if layout == "tbf":
+        out = torch.empty((T, B, F), dtype=torch.float32, device=dev)
+        post = out
+    else:
+        out = torch.empty((B, T, F), dtype=torch.float32, device=dev)
+        post = out.transpose(0, 1)
+    loss = torch.empty((T, B), dtype=torch.float32, device=dev)
+    nbytes = cabi.workspace_size(T, B, F, W.E, W.n_states)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    print(f"2^31: layout {layout} writer {writer} E={W.E} workspace {nbytes >> 20} MiB", flush=True)
+    cabi.set_dense_writer(writer)
+    try:
+        cabi.run_strided(am.data_ptr(), am.stride(0), am.stride(1), 0, d["edges"].data_ptr(), d["edges"].stride(0),
+                         d["w"].data_ptr(), d["se"].data_ptr(), d["se"].stride(0), d["lens"].data_ptr(), T, B, F, W.E,
+                         W.n_states, cabi.OUT_PROB, out.data_ptr(), post.stride(0), post.stride(1), loss.data_ptr(),
+                         ws.data_ptr(), nbytes, stream)
+        assert cabi.read_status(ws.data_ptr(), B, stream) == (0, -1)
+        assert cabi.last_dense_writer() == (1 if writer < 0 else 0)
+    finally:
+        cabi.set_dense_writer(-1)
+    valid = torch.arange(T, device=dev)[:, None] < d["lens"][None, :]
+    rowsum = post.sum(-1, dtype=torch.float64)
+    assert torch.all((rowsum[valid] - 1.0).abs() < 1e-4)
+    assert torch.all(rowsum[~valid] == 0)
+    allowed = torch.zeros((B, F), dtype=torch.bool, device=dev)
+    allowed[d["edges"][3].long(), d["edges"][2].long()] = True
+    assert torch.all(post.amax(0)[~allowed] == 0)
+    first = loss[0][None, :].expand_as(loss)
+    assert torch.all(((loss - first).abs() <= 1e-5 * first.abs())[valid])
+    _check_sequences_against_oracle(oracle, W, am, post, loss, [0, B // 2, B - 1])
+
+
+def test_best_path_more_than_2_to_31_elements(oracle):
+    """Best path over scores of 2.3e9 elements: alignments and scores of three sequences bit-identical to the oracle's,
+    every alignment entry an emission of its sequence."""
+    B = 192
+    W = make_workload("cart", B=B, with_am=False)
+    T, F = W.T, W.F
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(78)
+    am = torch.empty((T, B, F), dtype=torch.float32, device=dev)
+    for t0 in range(0, T, 50):
+        x = torch.randn((min(50, T - t0), B, F), generator=gen, device=dev) * 3.0
+        am[t0:t0 + 50] = torch.log_softmax(x.double(), -1).float()
+    del x
+    d = dict(edges=torch.from_numpy(W.edges).to(dev), w=torch.from_numpy(-W.weights).to(dev),
+             se=torch.from_numpy(W.start_end_states).to(dev), lens=torch.from_numpy(W.seq_lens).to(dev))
+    align = torch.empty((T, B), dtype=torch.int32, device=dev)
+    scores = torch.empty((B,), dtype=torch.float32, device=dev)
+    nbytes = cabi.workspace_size(T, B, F, W.E, W.n_states)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    print(f"2^31 best path: E={W.E}", flush=True)
+    cabi.viterbi(am.data_ptr(), am.stride(0), am.stride(1), d["edges"].data_ptr(), d["edges"].stride(0), d["w"].data_ptr(),
+                 d["se"].data_ptr(), d["se"].stride(0), d["lens"].data_ptr(), T, B, F, W.E, W.n_states,
+                 align.data_ptr(), align.stride(0), align.stride(1), scores.data_ptr(), ws.data_ptr(), nbytes, stream)
+    assert cabi.read_status(ws.data_ptr(), B, stream) == (0, -1)
+    allowed = torch.zeros((B, F), dtype=torch.bool, device=dev)
+    allowed[d["edges"][3].long(), d["edges"][2].long()] = True
+    valid = torch.arange(T, device=dev)[:, None] < d["lens"][None, :]
+    picked = allowed[torch.arange(B, device=dev)[None, :].expand(T, B), align.long().clamp(0, F - 1)]
+    assert torch.all(picked[valid])
+    which = np.array([0, B // 2, B - 1])
+    am_sub = np.ascontiguousarray(am[:, torch.from_numpy(which).to(dev), :].cpu().numpy())
+    keep = np.isin(W.edges[3], which)
+    edges = W.edges[:, keep].copy()
+    edges[3] = np.searchsorted(which, edges[3])
+    want_align, want_scores = oracle.viterbi_oracle(am_sub, edges, -W.weights[keep], W.start_end_states[:, which].copy(),
+                                                    W.seq_lens[which].copy(), W.n_states)
+    np.testing.assert_array_equal(align[:, torch.from_numpy(which).to(dev)].cpu().numpy(), want_align)
+    np.testing.assert_array_equal(scores.cpu().numpy()[which].view(np.uint32), want_scores.view(np.uint32))
