@@ -642,7 +642,8 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         m->S = (int)S; m->SP = SP; m->D = D; m->DP = DP; m->L = L;
         m->start_local = start_loc; m->end_local = end_loc;
         m->err = err ? err : (generic ? SEQ_GENERIC : 0);
-        // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered
+        // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered;
+        // bits 8 and up: see below
         m->pad = (sorted ? 1 : 0) | (sparse ? 2 : 0);
     }
     if (err || generic || n_edges == 0) {
@@ -788,6 +789,8 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         __syncthreads();
         dmax = s_dmax; dmin = s_dmin;
         const int s_loc = start_loc, e_loc = end_loc;
+        // for the recursion's renormalisation (see live_window): no edge lowers the state number, none raises it by more than dmax
+        if (tid == 0 && dmin == 0 && dmax > 0 && dmax < (1 << 20) && s_loc <= e_loc) a.meta[b].pad |= dmax << 8;
         // one thread per edge; the per-slot minimum / maximum is taken with LDS atomics in the
         // memory of the sort keys (and of the distinct ids of a renumbered sequence), which is not
         // needed any more once each thread has worked out the frames of its own edges
@@ -934,7 +937,57 @@ struct RecCursor {
     double c; bool pending;          // running offset, renormalisation requested by the last step
     int* progress; int nsteps;       // rows finished so far (SYNC), number of steps
     const int* gave_up;              // LDS word the loader wave sets when a wait of its own has run out
+    // for live_states: start and end state, largest rise of the state number along an edge (0: not known), frames,
+    // direction, and the two moving bounds for the row of the next group's last step
+    int live_s, live_e, live_d, live_L, live_dir, live_reach, live_left;
 };
+
+// The renormalisation takes the minimum over the states that can still lie on a path from the start
+// state to the end state: those reached from the start in at most p edges from which the end is at
+// most L - p edges away, p being the number of frames consumed by the row in question.  Without
+// this the minimum of a tightly constrained sequence sits at states that lag behind (cheap to stay
+// in, but too far from the end to matter), the states that carry the posterior mass are hundreds
+// of units above it, and their rows lose that much of float's precision (130 sequences of 991 states
+// over 1030 frames: posterior error 8.2e-5 before, 2.4e-5 with it).  Any offset is a valid one: the
+// states left out just end up below zero.
+// live_window: the steps whose row can hold state x on a complete path, as the first such step and the
+// number of further ones.  Known for automata whose edges never lower the state number (the
+// preparation then leaves the largest rise in the meta record, see min_steps); otherwise every
+// state counts in every step.  Two registers per state, and nothing for the scalar unit to carry
+// through the time loop.
+struct LiveWindow { int first; unsigned more; };
+__device__ __forceinline__ LiveWindow live_window(const SeqMeta& m, const int dir, const int x) {
+    const int d = m.pad >> 8, L = m.L;
+    LiveWindow all = { 0, 0x7fffffffu }, never = { 0x7fffffff, 0u };
+    if (d <= 0) return all;
+    if (x < m.start_local || x > m.end_local) return never;
+    const int plo = (x - m.start_local + d - 1) / d, phi = L - (m.end_local - x + d - 1) / d;    // frames consumed: plo <= p <= phi
+    // step i produces the row with p = i + 1 (alpha) or p = L - 1 - i (beta)
+    const int lo = max(0, dir ? L - 1 - phi : plo - 1), hi = dir ? L - 1 - plo : phi - 1;
+    if (hi < lo) return never;
+    LiveWindow w = { lo, (unsigned)(hi - lo) };
+    return w;
+}
+__device__ __forceinline__ bool is_live(const LiveWindow& w, const int i) { return (unsigned)(i - w.first) <= w.more; }
+// The same set seen from a step: the state numbers [lo, lo + span] that are live in the row it produces.
+// The instance with fifteen compute waves asks this way: it has no registers left for a window per state
+// (5 % of its time, measured), while scalar registers and the scalar unit are idle there; for the other
+// instances it is the other way round (a sequence of scalar operations in front of the wave minimum costs
+// a latency-bound step 4-6 %).
+template <int THREADS> struct LiveByStates { static constexpr bool value = THREADS == REC_THREADS_BIG; };
+struct LiveStates { int lo; unsigned span; };
+__device__ __forceinline__ LiveStates live_interval(const RecCursor& cur, const int reach, const int left) {
+    const int hi = min(cur.live_e, reach), lo = max(cur.live_s, left);
+    LiveStates r = { lo, hi >= lo ? (unsigned)(hi - lo) : 0u };
+    return r;
+}
+__device__ __forceinline__ LiveStates live_states(const RecCursor& cur, const int i) {
+    if (cur.live_d <= 0) { LiveStates all = { 0, 0x7fffffffu }; return all; }
+    const long long p = cur.live_dir ? cur.live_L - 1 - i : i + 1;      // frames consumed by the row step i produces
+    const long long reach = cur.live_s + p * cur.live_d, left = cur.live_e - (cur.live_L - p) * cur.live_d;
+    return live_interval(cur, (int)(reach < cur.live_e ? reach : cur.live_e), (int)(left > cur.live_s ? left : cur.live_s));
+}
+__device__ __forceinline__ bool is_live(const LiveStates& l, const int s) { return (unsigned)(s - l.lo) <= l.span; }
 
 // End of a step: the per-frame barrier and, every PUBLISH steps, the progress counter.  Stores
 // complete in issue order, so "at most PUBLISH of this wave's stores are still in flight" means
@@ -1014,7 +1067,7 @@ template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ>
 __device__ __forceinline__ void recurse_step(const int i, const int SP, const char* stc, ST* stn,
                                              const char* amc, float* wmin,
                                              const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
-                                             const float (&ew)[J][KT], RecCursor& cur) {
+                                             const float (&ew)[J][KT], const LiveWindow (&lw)[J], RecCursor& cur) {
     constexpr int NW = THREADS / 64;
     const int tid = threadIdx.x;
     float pend = 0.f;
@@ -1025,7 +1078,7 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         pend = mn == INF_F ? 0.f : mn;
         cur.c += (double)pend;
     }
-    float rmin = INF_F;
+    float rj[NJ > 0 ? NJ : 1];
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
         const int s = tid + j * THREADS;
@@ -1035,12 +1088,18 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
         const ST r = state_value<KT, ST, true>(v, pend);
         stn[s] = r;
         if (s < SP) store_x<SYNC>(cur.wp + s, (float)r);
-        rmin = fminf(rmin, (float)r);
+        rj[j] = (float)r;
     }
     if (tid == 0) store_x<SYNC>(cur.op, cur.c);
     cur.wp += cur.wstep; cur.op += cur.ostep;
     cur.pending = (i % RENORM) == RENORM - 1;
     if (cur.pending) {
+        float rmin = INF_F;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const bool live = LiveByStates<THREADS>::value ? is_live(live_states(cur, i), tid + j * THREADS) : is_live(lw[j], i);
+            rmin = fminf(rmin, live ? rj[j] : INF_F);
+        }
         rmin = wave_min_dpp(rmin);
         if ((tid & 63) == 63) wmin[tid >> 6] = rmin;
     }
@@ -1054,9 +1113,9 @@ __device__ __forceinline__ void recurse_step(const int i, const int SP, const ch
 // row store and the barrier (which the caller issues): the recursion is bound by the number of
 // instructions a SIMD has to issue per frame for the waves it holds.
 template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ, bool FIRST, bool LAST>
-__device__ __forceinline__ void recurse_step_in_group(const int SP, const char* stc, ST* stn, const char* amc, float* wmin,
+__device__ __forceinline__ void recurse_step_in_group(const int i, const int SP, const char* stc, ST* stn, const char* amc, float* wmin,
                                                       const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
-                                                      const float (&ew)[J][KT], RecCursor& cur) {
+                                                      const float (&ew)[J][KT], const LiveWindow (&lw)[J], RecCursor& cur) {
     constexpr int NW = THREADS / 64;
     const int tid = threadIdx.x;
     float pend = 0.f;
@@ -1070,6 +1129,14 @@ __device__ __forceinline__ void recurse_step_in_group(const int SP, const char* 
         cur.op += RENORM * cur.ostep;
     }
     float rmin = INF_F;
+    LiveStates states = { 0, 0u };
+    if (LAST && LiveByStates<THREADS>::value) {
+        // (the two bounds move by RENORM frames from one group to the next; a sequence long enough for them to leave the
+        // range of int has had its live_d set to 0 by recurse_init)
+        states = live_interval(cur, cur.live_reach, cur.live_left);
+        const int inc = (cur.live_dir ? -RENORM : RENORM) * cur.live_d;
+        cur.live_reach += inc; cur.live_left += inc;
+    }
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
         const int s = tid + j * THREADS;
@@ -1079,7 +1146,7 @@ __device__ __forceinline__ void recurse_step_in_group(const int SP, const char* 
         const ST r = state_value<KT, ST, FIRST>(v, pend);
         stn[s] = r;
         if (s < SP) store_x<SYNC>(cur.wp + s, (float)r);
-        if (LAST) rmin = fminf(rmin, (float)r);
+        if (LAST) rmin = fminf(rmin, (LiveByStates<THREADS>::value ? is_live(states, s) : is_live(lw[j], i)) ? (float)r : INF_F);
     }
     cur.wp += cur.wstep;
     if (LAST) {
@@ -1092,7 +1159,7 @@ __device__ __forceinline__ void recurse_step_in_group(const int SP, const char* 
 template <bool SYNC, int THREADS, int J, int KT, typename ST, int NJ>
 __device__ __forceinline__ void recurse_time_loop(const int SP, ST* st0, ST* st1, const float* am0, const float* am1, float* wmin,
                                                   const unsigned (&eo)[J][KT], const unsigned (&es)[J][KT],
-                                                  const float (&ew)[J][KT], RecCursor& cur) {
+                                                  const float (&ew)[J][KT], const LiveWindow (&lw)[J], RecCursor& cur) {
     static_assert(RENORM == 8 && PUBLISH % RENORM == 0, "shape of a group of steps");
     const char* c0 = (const char*)st0; const char* c1 = (const char*)st1;
     const char* a0 = (const char*)am0; const char* a1 = (const char*)am1;
@@ -1105,19 +1172,19 @@ __device__ __forceinline__ void recurse_time_loop(const int SP, ST* st0, ST* st1
             g_trace[64 + (blockIdx.x < 2 ? blockIdx.x : 2 + (blockIdx.x & 1)) * 64 + 32 + i / 48] = clock64();
         }
 #endif
-        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, true, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, true, false>(i, SP, c0, st1, a0, wmin, eo, es, ew, lw, cur);
         lds_barrier();
-        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(i, SP, c1, st0, a1, wmin, eo, es, ew, lw, cur);
         lds_barrier();
         for (int r = 0; r < (RENORM - 4) / 2; r++) {
-            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(i, SP, c0, st1, a0, wmin, eo, es, ew, lw, cur);
             lds_barrier();
-            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+            recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(i, SP, c1, st0, a1, wmin, eo, es, ew, lw, cur);
             lds_barrier();
         }
-        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(SP, c0, st1, a0, wmin, eo, es, ew, cur);
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, false>(i, SP, c0, st1, a0, wmin, eo, es, ew, lw, cur);
         lds_barrier();
-        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, true>(SP, c1, st0, a1, wmin, eo, es, ew, cur);
+        recurse_step_in_group<SYNC, THREADS, J, KT, ST, NJ, false, true>(i + RENORM - 1, SP, c1, st0, a1, wmin, eo, es, ew, lw, cur);
         // as step_end for the step i + RENORM - 1, which is never the last one
         const bool pub = SYNC && ((i + RENORM) % PUBLISH) == 0;
         static_assert(PUBLISH == 32, "the wait count below is PUBLISH");
@@ -1128,9 +1195,9 @@ __device__ __forceinline__ void recurse_time_loop(const int SP, ST* st0, ST* st1
     cur.pending = i > 0;
     // the rest, at most RENORM steps, the last one among them
     for (; i < cur.nsteps; i += 2) {
-        recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i, SP, c0, st1, a0, wmin, eo, es, ew, cur);
+        recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i, SP, c0, st1, a0, wmin, eo, es, ew, lw, cur);
         if (i + 1 < cur.nsteps)
-            recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i + 1, SP, c1, st0, a1, wmin, eo, es, ew, cur);
+            recurse_step<SYNC, THREADS, J, KT, ST, NJ>(i + 1, SP, c1, st0, a1, wmin, eo, es, ew, lw, cur);
     }
 }
 
@@ -1164,6 +1231,14 @@ __device__ __forceinline__ void recurse_init(const RecArgs& a, const SeqMeta& m,
     cur.progress = a.sync + SYNC_HDR + 2 * b + dir;
     cur.gave_up = rec_gave_up(wmin);
     cur.nsteps = L - 1;
+    cur.live_s = m.start_local; cur.live_e = m.end_local; cur.live_L = L; cur.live_dir = dir;
+    cur.live_d = (long long)(m.pad >> 8) * L < (1 << 30) ? m.pad >> 8 : 0;
+    if (cur.live_d > 0) {
+        const int p = dir ? L - RENORM : RENORM;       // frames consumed by the row of step RENORM - 1, the first to ask
+        cur.live_reach = cur.live_s + p * cur.live_d; cur.live_left = cur.live_e - (L - p) * cur.live_d;
+    } else {
+        cur.live_s = 0; cur.live_e = 0x7fffffff; cur.live_reach = 0x7fffffff; cur.live_left = 0;
+    }
     if (SYNC) wait_stores();
     lds_barrier();
     if (SYNC && tid == 0) store_agent(cur.progress, 1);      // the initial row is out
@@ -1198,6 +1273,12 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
             ew[j][k] = __uint_as_float(r.y);
         }
     }
+    LiveWindow lw[J];
+#pragma unroll
+    for (int j = 0; j < J; j++) {
+        if (LiveByStates<THREADS>::value) { lw[j].first = 0; lw[j].more = 0u; }      // not used: see live_states
+        else lw[j] = live_window(m, dir, tid + j * THREADS);
+    }
     if (tid < THREADS / 64) wmin[tid] = INF_F;
     RecCursor cur;
     recurse_init<SYNC, THREADS, ST>(a, m, b, dir, SCAP, st0, st1, wmin, cur);
@@ -1212,11 +1293,11 @@ __device__ __forceinline__ void recurse_compute(const RecArgs& a, const SeqMeta&
     // (only in the instance for small batches: the one of which two workgroups share a compute unit
     // has no registers to spare for more loop bodies)
     constexpr bool PER_ROUND = THREADS == REC_THREADS || THREADS == REC_THREADS_BIG;
-    if (!PER_ROUND) recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
-    else if (J == 1 || nj == 1) recurse_time_loop<SYNC, THREADS, J, KT, ST, 1>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
-    else if (nj == 2) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 2 ? 2 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
-    else if (nj == 3) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 3 ? 3 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
-    else recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, cur);
+    if (!PER_ROUND) recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, lw, cur);
+    else if (J == 1 || nj == 1) recurse_time_loop<SYNC, THREADS, J, KT, ST, 1>(SP, st0, st1, am0, am1, wmin, eo, es, ew, lw, cur);
+    else if (nj == 2) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 2 ? 2 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, lw, cur);
+    else if (nj == 3) recurse_time_loop<SYNC, THREADS, J, KT, ST, (J >= 3 ? 3 : 1)>(SP, st0, st1, am0, am1, wmin, eo, es, ew, lw, cur);
+    else recurse_time_loop<SYNC, THREADS, J, KT, ST, J>(SP, st0, st1, am0, am1, wmin, eo, es, ew, lw, cur);
 }
 
 // Fallback for the largest sequences: same arithmetic, edge tables re-read from memory each frame
@@ -1246,6 +1327,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
             cur.c += (double)pend;
         }
         float rmin = INF_F;
+        const bool want_min = (i % RENORM) == RENORM - 1;       // over the states that still matter, see live_window
         if (K > KMAX) {
             // degree beyond the unrolled body: two passes over the state's table column
             for (int s = tid; s < SP; s += THREADS) {
@@ -1261,7 +1343,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
                 const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
                 stn[s] = r;
                 store_x<SYNC>(cur.wp + s, (float)r);
-                rmin = fminf(rmin, (float)r);
+                if (want_min && is_live(live_window(m, dir, s), i)) rmin = fminf(rmin, (float)r);
             }
         } else
         for (int s = tid; s < SP; s += THREADS) {
@@ -1283,7 +1365,7 @@ __device__ __forceinline__ void recurse_compute_generic(const RecArgs& a, const 
             const ST r = mn == (ST)INF_F ? (ST)INF_F : (mn - (ST)pend) - (ST)__builtin_amdgcn_logf(sum);
             stn[s] = r;
             store_x<SYNC>(cur.wp + s, (float)r);
-            rmin = fminf(rmin, (float)r);
+            if (want_min && is_live(live_window(m, dir, s), i)) rmin = fminf(rmin, (float)r);
         }
         if (tid == 0) store_x<SYNC>(cur.op, cur.c);
         cur.wp += cur.wstep; cur.op += cur.ostep;
