@@ -40,7 +40,8 @@ enum {
 /* Layout of the posterior tensor written by i6fbw_run. */
 enum {
     I6FBW_OUT_NEG_LOG = 0,   /* -log posterior, +inf where nothing contributes: what fbw_core.fbw returns
-                                (fbw_op.cu:366-377,392) */
+                                (fbw_op.cu:366-377,392); finite wherever some edge contributes, however little
+                                (also for posteriors far below float's range: the reference adds in log space) */
     I6FBW_OUT_PROB = 1,      /* posterior itself, 0 where nothing contributes: what
                                 FastBaumWelchLoss.backward derives from it (fbw/__init__.py:40-44) */
     I6FBW_OUT_NEG_PROB = 2   /* minus the posterior: the gradient that reaches `log_probs` in fbw_loss

@@ -24,8 +24,11 @@ def check_against_oracle(oracle, args, threads=1, bitwise=True):
     np.testing.assert_allclose(loss, want_loss, rtol=LOSS_RTOL, atol=1e-6)
     assert (loss[want_loss == 0] == 0).all()
     np.testing.assert_allclose(posterior(out), want_post, rtol=0, atol=POST_ATOL)
-    # holes are +inf in exactly the same places (a posterior below float range may differ)
-    assert (np.isposinf(out) | (want_post < 1e-30) == np.isposinf(want_out) | (want_post < 1e-30)).all()
+    # holes are +inf in exactly the same places -- also where a posterior is below float's range: the reference adds in
+    # log space (fbw_op.cu:115-134) and has a finite -log there -- and the finite values agree in the log domain too
+    fin = np.isfinite(want_out)
+    assert (np.isposinf(out) == ~fin).all()
+    np.testing.assert_allclose(out[fin], want_out[fin], rtol=2e-5, atol=2e-3)
     prob, loss2 = run_cabi(*args, out_mode=cabi.OUT_PROB)
     if bitwise:      # the fast kernels sum in a fixed order; the general path accumulates with atomics
         np.testing.assert_array_equal(loss2, loss)
