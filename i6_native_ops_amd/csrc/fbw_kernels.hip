@@ -3039,6 +3039,10 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // All 2B recursion workgroups must be on the machine at the same time (at most two per compute
     // unit): gather and dense write wait for their progress while occupying wave slots themselves.
     if (2 * B > (dense ? 2 : 1) * P.n_cu) overlap = false;
+    // (a workgroup of the instance for large automata fills the register file of its compute unit: the kernels it
+    // waits for need units of their own -- with 240 such workgroups on 256 units a forced overlap ran into the bound
+    // of its waits)
+    if (big && 2 * B > P.n_cu / 2) overlap = false;
     // Two workgroups of the dense instance are four waves per SIMD: beyond 104 registers each they
     // leave no room for the gather's waves, which they wait for.  (The compiler is asked for 96; how
     // close it gets depends on its version.)

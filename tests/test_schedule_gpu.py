@@ -91,3 +91,23 @@ def test_waits_that_run_out_leave_nan_and_a_status(writer):
     out2, loss2 = P.run(cabi.OUT_PROB)
     np.testing.assert_array_equal(out2.cpu().numpy(), good_out)
     np.testing.assert_array_equal(loss2.cpu().numpy(), good_loss)
+
+
+def test_forced_overlap_with_a_unit_filling_workgroup_per_sequence(oracle):
+    """100 chains of 541 states: the recursion instance for large automata, whose workgroups fill a compute
+    unit's register file each.  Asked for the overlapped schedule the library declines (200 such workgroups would
+    leave the kernels they wait for a fifth of the device, and the waits ran into their bound): the call must
+    succeed and equal the oracle either way."""
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import run_cabi
+    W = make_workload("cart", seed=41, T=640, B=100, F=40, n_labels=(180, 180))
+    args = (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    assert W.n_states > 512 * W.B
+    want_out, want_loss = oracle.fbw_oracle(*args, threads=16)
+    cabi.set_overlap(1)
+    try:
+        out, loss = run_cabi(*args, out_mode=cabi.OUT_PROB)      # raises on a device-side status
+    finally:
+        cabi.set_overlap(-1)
+    np.testing.assert_allclose(loss, want_loss, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(out, posterior(want_out), rtol=0, atol=1e-4)
