@@ -1755,34 +1755,6 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-// -log of a slot's posterior.  Where the slot's share of the frame's mass, taken relative to the frame
-// minimum as everywhere else, is below 2^-100, the sums lose their terms to float's range (flushed to
-// zero below 2^-126) -- while the reference, which adds in log space (fbw_op.cu:115-134), still has a
-// finite value there: such a slot's edges are taken once more, from memory, relative to the slot's own
-// minimum.  Rare (posteriors below 1e-30) and only in the -log output.
-constexpr float TINY_SLOT = 7.888609e-31f;      // 2^-100
-template <bool SYNC>
-__device__ __noinline__ float tiny_slot_neg_log(const uint4* crec, const int e0, const int e1, const float* arow, const float* brow,
-                                                const float* grow, const float mn, const float logtot) {
-    auto score = [&](int i) {
-        const uint4 r = crec[i];
-        return (load_x<SYNC>(arow + (r.x & 0xFFFFu)) + __uint_as_float(r.y)) + (load_x<SYNC>(grow + r.z) + load_x<SYNC>(brow + (r.x >> 16)));
-    };
-    float smin = INF_F;
-    for (int i = e0; i < e1; i++) smin = fminf(smin, score(i));
-    if (!(smin < INF_F)) return INF_F;           // no edge of the slot is alive in this frame: a hole
-    float sum = 0.f;
-    for (int i = e0; i < e1; i++) sum += __builtin_amdgcn_exp2f(smin - score(i));
-    return (logtot - ((mn - smin) + __builtin_amdgcn_logf(sum))) * LN2;
-}
-template <bool SYNC>
-__device__ __forceinline__ float slot_neg_log(const bool dead, const float sd, const float logtot, const float mn, const uint4* crec,
-                                              const int* cbd, const float* arow, const float* brow, const float* grow) {
-    if (dead) return INF_F;
-    if (sd >= TINY_SLOT) return (logtot - __builtin_amdgcn_logf(sd)) * LN2;
-    return tiny_slot_neg_log<SYNC>(crec, cbd[0], cbd[1], arow, brow, grow, mn, logtot);       // cbd: the slot's entry of the CSR index
-}
-
 // Sum of xs[c0, c1), every lane with a range of its own; called by whole waves.  Ranges of up to
 // LONG_SLOT entries are summed by their lane.  Longer ones (the blank label of a CTC automaton,
 // silence: one emission class on a large share of the edges) would keep one lane busy for
@@ -1918,7 +1890,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             // their positions get the hole value back.
             auto value = [&](int js) -> float {
                 if (prob) return sd[js] * inv;
-                return slot_neg_log<SYNC>(dead, sd[js], logtot, mn, crec, cb + tid + js * COMB_THREADS, abase + (size_t)t * SP, bbase + (size_t)t * SP, gbase + (size_t)t * DP);
+                return (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
             };
             float* base = orow - sh;
             const int W = a.tile_w, P = sh + F;
@@ -1955,7 +1927,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             if (d < D) {
                 float v;
                 if (prob) v = sd[js] * inv;
-                else v = slot_neg_log<SYNC>(dead, sd[js], logtot, mn, crec, cb + d, abase + (size_t)t * SP, bbase + (size_t)t * SP, gbase + (size_t)t * DP);
+                else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
                 image[sh + em[js]] = v;
             }
         }
@@ -2332,7 +2304,7 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
                 if (d < D) {
                     float v;
                     if (prob) v = sd[js] * inv;
-                    else v = slot_neg_log<SYNC>(dead, sd[js], logtot, mn, crec, cb + d, abase + (size_t)t * SP, bbase + (size_t)t * SP, gbase + (size_t)t * DP);
+                    else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
                     store_agent(cprow + d, v);
                 }
             }
@@ -2406,7 +2378,7 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
             if (d < D) {
                 float v;
                 if (prob) v = sd[js] * inv;
-                else v = slot_neg_log<SYNC>(dead, sd[js], logtot, mn, crec, cb + d, abase + (size_t)t * SP, bbase + (size_t)t * SP, gbase + (size_t)t * DP);
+                else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
                 store_agent(cprow + d, v);
             }
         }

@@ -40,8 +40,9 @@ enum {
 /* Layout of the posterior tensor written by i6fbw_run. */
 enum {
     I6FBW_OUT_NEG_LOG = 0,   /* -log posterior, +inf where nothing contributes: what fbw_core.fbw returns
-                                (fbw_op.cu:366-377,392); finite wherever some edge contributes, however little
-                                (also for posteriors far below float's range: the reference adds in log space) */
+                                (fbw_op.cu:366-377,392).  Also +inf where the posterior is below float's range (about
+                                1e-38: a -log above 87, where the reference, which adds in log space, still has a
+                                finite value) */
     I6FBW_OUT_PROB = 1,      /* posterior itself, 0 where nothing contributes: what
                                 FastBaumWelchLoss.backward derives from it (fbw/__init__.py:40-44) */
     I6FBW_OUT_NEG_PROB = 2   /* minus the posterior: the gradient that reaches `log_probs` in fbw_loss
