@@ -24,11 +24,45 @@ def _run(cmd):
     subprocess.check_call(cmd)
 
 
+def kernel_resources(remarks):
+    """{kernel name: {"vgprs": n, "scratch": bytes per lane, "occupancy": waves per SIMD}} from the compiler's
+    kernel-resource-usage remarks"""
+    import re
+    out, cur = {}, None
+    for line in remarks.splitlines():
+        m = re.search(r"remark: Function Name: (\S+)", line)
+        if m:
+            cur = out.setdefault(m.group(1), {})
+            continue
+        for key, pat in (("vgprs", r"remark:\s+VGPRs: (\d+)"), ("scratch", r"ScratchSize \[bytes/lane\]: (\d+)"),
+                         ("occupancy", r"Occupancy \[waves/SIMD\]: (\d+)")):
+            m = re.search(pat, line)
+            if m and cur is not None:
+                cur[key] = int(m.group(1))
+    return out
+
+
 def build_lib(out_root=PKG):
-    """libi6fbw.so into <out_root>/fbw (out_root: this package in the source tree, or its copy in a build tree)"""
+    """libi6fbw.so into <out_root>/fbw (out_root: this package in the source tree, or its copy in a build tree),
+    and beside it kernel_resources.json: registers, scratch and occupancy of every kernel as the compiler reports
+    them (a kernel that outgrows its register budget spills without a word and runs at half its speed;
+    tests/test_boundary_cpu.py reads this record)."""
+    import json
     lib = os.path.join(out_root, "fbw", "libi6fbw.so")
     os.makedirs(os.path.dirname(lib), exist_ok=True)
-    _run([HIPCC, *HIP_FLAGS, "-shared", os.path.join(CSRC, "fbw_kernels.hip"), "-o", lib])
+    cmd = [HIPCC, *HIP_FLAGS, "-shared", "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, "fbw_kernels.hip"), "-o", lib]
+    print(" ".join(cmd), flush=True)
+    done = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    remarks = done.stdout
+    import re
+    other = [l for l in remarks.splitlines()
+             if "-Rpass-analysis=kernel-resource-usage" not in l and not re.match(r"^\s*(\d+ )?\|", l)]     # (and the source lines quoted with them)
+    if other:
+        print("\n".join(other), flush=True)
+    if done.returncode != 0:
+        raise subprocess.CalledProcessError(done.returncode, cmd)
+    with open(os.path.join(out_root, "fbw", "kernel_resources.json"), "w") as f:
+        json.dump(kernel_resources(remarks), f, indent=1, sort_keys=True)
     return lib
 
 

@@ -109,3 +109,32 @@ def test_packaging_metadata():
     from i6_native_ops_amd import build
     import inspect
     assert "out_root" in inspect.signature(build.build_all).parameters
+
+
+def test_kernels_stay_within_their_register_budgets():
+    """The build records what the compiler reports for every kernel.  The dense writer is launched for eight waves per
+    SIMD (64 registers) and the gather, the preparation and the recursion instance for small batches are written to
+    need no scratch memory: a change that pushes one of them over its budget makes the compiler spill without a word
+    (the dense write of the CTC configuration once went from 0.19 to 0.37 ms that way)."""
+    import json
+    import os
+    from i6_native_ops_amd import cabi
+    path = os.path.join(os.path.dirname(cabi.LIB_PATH), "kernel_resources.json")
+    if not os.path.exists(path):
+        pytest.skip("kernel_resources.json is written by `python -m i6_native_ops_amd.build`")
+    res = json.load(open(path))
+
+    def kernels(fragment):
+        found = {k: v for k, v in res.items() if fragment in k}
+        assert found, fragment
+        return found
+
+    for name, r in kernels("fbw_flat").items():
+        assert r["scratch"] == 0 and r["vgprs"] <= 64 and r["occupancy"] == 8, (name, r)
+    for fragment in ("fbw_gather", "fbw_prepare", "fbw_padfill", "fbw_scan_sorted", "11fbw_recurseI", "vit_align"):
+        for name, r in kernels(fragment).items():
+            assert r["scratch"] == 0, (name, r)
+    for name, r in kernels("fbw_recurse_dense").items():
+        assert r["vgprs"] <= 104, (name, r)          # two workgroups per compute unit and room for the gather's waves
+    for name, r in kernels("fbw_recurse_big").items():
+        assert r["vgprs"] <= 128, (name, r)          # sixteen waves per compute unit
