@@ -2098,6 +2098,74 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// -log output only: posteriors below float's range.  The kernels above sum a slot's probabilities
+// relative to the frame minimum; a slot whose share is below 2^-126 of that flushes to zero and its
+// element comes out as +inf, while the reference, which adds in log space (fbw_op.cu:115-134), has
+// a finite value there (a -log above 87).  This pass goes over the elements of the emissions a
+// sequence uses, frame by frame, after the dense write: where one holds +inf although an edge of its
+// slot is alive -- or a value so large that its sum may have lost terms --, the slot is summed once more relative
+// to its own minimum,
+//     -log p = ln 2 * (min_e x_e - log2 sum_e 2^(min - x_e) + row offsets) - loss,
+// with the frame's loss as the dense write left it.  A pass of its own, because the same lines
+// inside fbw_flat cost that kernel its register budget (and the dense write half its speed).  Sequences
+// on the general path add in log space anyway.  About as much traffic as the gather, in this output
+// mode only.
+// ---------------------------------------------------------------------------------------------
+constexpr int TAIL_FRAMES = 8;
+// (the emission scores from am_scores themselves, as the gather scales them: by now the compact table may hold the flat
+// writer's values)
+// cp: the flat writer's compact values [seq][t][slot] (what it copied into the tensor; read in place of the tensor's
+// scattered elements for the sequences it wrote), or null.
+__global__ __launch_bounds__(COMB_THREADS) void fbw_neg_log_tail(CombArgs a, const float* am, long long st_t, long long st_b, float scale,
+                                                                 const float* cp) {
+    const int b = blockIdx.y, t0 = blockIdx.x * TAIL_FRAMES, tid = threadIdx.x;
+    const SeqMeta m = a.meta[b];
+    if (rec_class(m) <= 0) return;
+    const int nt = min(m.L, t0 + TAIL_FRAMES) - t0;
+    if (nt <= 0) return;
+    const int D = m.D, SP = m.SP, DP = m.DP;
+    const long long soff = state_off(m.edge_begin, b), goff = slot_off(m.edge_begin, b);
+    const uint4* crec = a.crec + m.edge_begin;
+    const int* cb = a.cbegin + goff;
+    const int* de = a.demis + goff;
+    const float* compact = (cp && flat_fast(m)) ? cp + (size_t)a.T * goff : nullptr;
+    for (int d = tid; d < D; d += COMB_THREADS) {
+        const int em = de[d];
+        // the values of all frames first: the loads are in flight together
+        float v[TAIL_FRAMES];
+#pragma unroll
+        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
+            v[tt] = 0.f;
+            if (tt < nt) v[tt] = compact ? compact[(size_t)(t0 + tt) * DP + d] : a.out[(t0 + tt) * a.ost_t + b * a.ost_b + em];
+        }
+#pragma unroll
+        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
+            // (not only +inf: from 2^-100 of the frame minimum down a sum may have lost some of its terms; as a -log
+            // that is 69 and more, whatever the frame's normaliser, which is at least 1)
+            if (!(v[tt] > 69.f)) continue;
+            const int t = t0 + tt;
+            const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
+            const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
+            const float* amrow = am + (long long)t * st_t + (long long)b * st_b;
+            auto score = [&](int i) {
+                const uint4 r = crec[i];
+                const float g = amrow[de[r.z]];
+                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + ((g == INF_F ? INF_F : g * scale) + brow[r.x >> 16]);      // as in fbw_gather and fbw_combine
+            };
+            const int e0 = cb[d], e1 = cb[d + 1];
+            float smin = INF_F;
+            for (int i = e0; i < e1; i++) smin = fminf(smin, score(i));
+            if (!(smin < INF_F)) continue;                    // a hole: no edge of the slot is alive in this frame
+            float sum = 0.f;
+            for (int i = e0; i < e1; i++) sum += __builtin_amdgcn_exp2f(smin - score(i));
+            const double offs = a.offA[(size_t)b * a.T + t] + a.offB[(size_t)b * a.T + t];
+            const double loss = (double)a.sum_output[(size_t)t * a.B + b];
+            a.out[t * a.ost_t + b * a.ost_b + em] = (float)((((double)smin - (double)__builtin_amdgcn_logf(sum)) + offs) * (double)LN2 - loss);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // stage 4, flat form (fbw_flat).  The dense tensor is mostly holes: of the 12001 floats of a row of
 // the headline workload about 370 carry a posterior.  Here the posteriors of a frame are first
 // computed in compact form (one float per distinct emission of the sequence), and the tensor is
@@ -3061,6 +3129,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     ca.tile_w = tiled ? COMB_TILE_W : 0;
     ca.direct_only = 0;
+    const dim3 tail_grid((unsigned)((T + TAIL_FRAMES - 1) / TAIL_FRAMES), (unsigned)B);
     // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
     // order of frames and sequences, rows are long enough for a span to cut at most two of them,
     // and the tensor is large (for small problems the row writer is as good).
@@ -3172,6 +3241,10 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
             { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_flat<false>, dim3((unsigned)flat_grid), dim3(COMB_THREADS), 0, s, fa); }
         } else { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
         HIP_TRY(hipGetLastError());
+        if (out_mode == I6FBW_OUT_NEG_LOG) {
+            hipLaunchKernelGGL(fbw_neg_log_tail, tail_grid, dim3(COMB_THREADS), 0, s, ca, ga.am, ga.st_t, ga.st_b, ga.scale, flat ? (const float*)fa.cp : (const float*)nullptr);
+            HIP_TRY(hipGetLastError());
+        }
         return I6FBW_OK;
     }
 
@@ -3212,6 +3285,10 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     join_guard.joined = true;
+    if (out_mode == I6FBW_OUT_NEG_LOG) {
+        hipLaunchKernelGGL(fbw_neg_log_tail, tail_grid, dim3(COMB_THREADS), 0, s, ca, ga.am, ga.st_t, ga.st_b, ga.scale, flat ? (const float*)fa.cp : (const float*)nullptr);
+        HIP_TRY(hipGetLastError());
+    }
     return I6FBW_OK;
 }
 }  // namespace

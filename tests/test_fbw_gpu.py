@@ -24,14 +24,12 @@ def check_against_oracle(oracle, args, threads=1, bitwise=True):
     np.testing.assert_allclose(loss, want_loss, rtol=LOSS_RTOL, atol=1e-6)
     assert (loss[want_loss == 0] == 0).all()
     np.testing.assert_allclose(posterior(out), want_post, rtol=0, atol=POST_ATOL)
-    # holes are +inf in exactly the same places, and the finite values agree in the log domain too.  Posteriors below
-    # float's range are the exception: the reference adds in log space (fbw_op.cu:115-134) and has a finite -log
-    # above 87 there, this library sums probabilities relative to the frame minimum and writes +inf.
+    # holes are +inf in exactly the same places -- also where a posterior is below float's range: the reference adds in
+    # log space (fbw_op.cu:115-134) and has a finite -log there -- and the finite values agree in the log domain too
     fin = np.isfinite(want_out)
-    sure = want_post >= 1e-30
-    assert (np.isposinf(out) | ~sure == ~fin | ~sure).all()
-    assert not np.isfinite(out[~fin]).any()
-    np.testing.assert_allclose(out[fin & sure], want_out[fin & sure], rtol=2e-5, atol=2e-3)
+    assert (np.isposinf(out) == ~fin).all()
+    # (a -log above 69 is the difference of two numbers of the size of the loss, which is a float: half an ulp of it on top)
+    np.testing.assert_allclose(out[fin], want_out[fin], rtol=2e-5, atol=2e-3 + 1.2e-7 * float(np.abs(want_loss).max()))
     prob, loss2 = run_cabi(*args, out_mode=cabi.OUT_PROB)
     if bitwise:      # the fast kernels sum in a fixed order; the general path accumulates with atomics
         np.testing.assert_array_equal(loss2, loss)
