@@ -2132,11 +2132,14 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_neg_log_tail(CombArgs a, con
     for (int d = tid; d < D; d += COMB_THREADS) {
         const int em = de[d];
         // the values of all frames first: the loads are in flight together
-        float v[TAIL_FRAMES];
+        float v[TAIL_FRAMES], g[TAIL_FRAMES];       // and the slot's emission score in each of them (all edges of a slot share it)
 #pragma unroll
         for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            v[tt] = 0.f;
-            if (tt < nt) v[tt] = compact ? compact[(size_t)(t0 + tt) * DP + d] : a.out[(t0 + tt) * a.ost_t + b * a.ost_b + em];
+            v[tt] = 0.f; g[tt] = INF_F;
+            if (tt < nt) {
+                v[tt] = compact ? compact[(size_t)(t0 + tt) * DP + d] : a.out[(t0 + tt) * a.ost_t + b * a.ost_b + em];
+                g[tt] = __builtin_nontemporal_load(&am[(long long)(t0 + tt) * st_t + (long long)b * st_b + em]);
+            }
         }
 #pragma unroll
         for (int tt = 0; tt < TAIL_FRAMES; tt++) {
@@ -2146,11 +2149,10 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_neg_log_tail(CombArgs a, con
             const int t = t0 + tt;
             const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
             const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
-            const float* amrow = am + (long long)t * st_t + (long long)b * st_b;
+            const float gs = g[tt] == INF_F ? INF_F : g[tt] * scale;          // as fbw_gather scales it
             auto score = [&](int i) {
                 const uint4 r = crec[i];
-                const float g = amrow[de[r.z]];
-                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + ((g == INF_F ? INF_F : g * scale) + brow[r.x >> 16]);      // as in fbw_gather and fbw_combine
+                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + (gs + brow[r.x >> 16]);      // as in fbw_combine
             };
             const int e0 = cb[d], e1 = cb[d + 1];
             float smin = INF_F;
