@@ -2133,36 +2133,67 @@ __global__ __launch_bounds__(COMB_THREADS) void fbw_neg_log_tail(CombArgs a, con
         const int em = de[d];
         // the values of all frames first: the loads are in flight together
         float v[TAIL_FRAMES], g[TAIL_FRAMES];       // and the slot's emission score in each of them (all edges of a slot share it)
+        double base[TAIL_FRAMES];                   // row offsets * ln 2 - loss of the frame
 #pragma unroll
         for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            v[tt] = 0.f; g[tt] = INF_F;
+            v[tt] = 0.f; g[tt] = INF_F; base[tt] = 0.0;
             if (tt < nt) {
+                base[tt] = (a.offA[(size_t)b * a.T + t0 + tt] + a.offB[(size_t)b * a.T + t0 + tt]) * (double)LN2
+                           - (double)a.sum_output[(size_t)(t0 + tt) * a.B + b];
                 v[tt] = compact ? compact[(size_t)(t0 + tt) * DP + d] : a.out[(t0 + tt) * a.ost_t + b * a.ost_b + em];
                 g[tt] = __builtin_nontemporal_load(&am[(long long)(t0 + tt) * st_t + (long long)b * st_b + em]);
             }
         }
+        // (not only +inf: from 2^-100 of the frame minimum down a sum may have lost some of its terms; as a -log
+        // that is 69 and more, whatever the frame's normaliser, which is at least 1)
+        bool any = false;
+#pragma unroll
+        for (int tt = 0; tt < TAIL_FRAMES; tt++) any |= v[tt] > 69.f;
+        if (!any) continue;
+        const int e0 = cb[d], e1 = cb[d + 1];
+        constexpr int NE = 4;                 // edges of a slot held in registers (the usual slot has one or two)
+        uint4 r[NE];
+#pragma unroll
+        for (int k = 0; k < NE; k++) r[k] = e0 + k < e1 ? crec[e0 + k] : make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);      // weight +inf: contributes nothing
+        const bool few = e1 - e0 <= NE;
+        // the row elements of all frames and edges first (in flight together), then the arithmetic
+        float xa[TAIL_FRAMES][NE], xb[TAIL_FRAMES][NE];
 #pragma unroll
         for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            // (not only +inf: from 2^-100 of the frame minimum down a sum may have lost some of its terms; as a -log
-            // that is 69 and more, whatever the frame's normaliser, which is at least 1)
-            if (!(v[tt] > 69.f)) continue;
             const int t = t0 + tt;
             const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
             const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
+#pragma unroll
+            for (int k = 0; k < NE; k++) {
+                xa[tt][k] = INF_F; xb[tt][k] = INF_F;
+                if (few && v[tt] > 69.f && e0 + k < e1) { xa[tt][k] = arow[r[k].x & 0xFFFFu]; xb[tt][k] = brow[r[k].x >> 16]; }
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
+            if (!(v[tt] > 69.f)) continue;
+            const int t = t0 + tt;
             const float gs = g[tt] == INF_F ? INF_F : g[tt] * scale;          // as fbw_gather scales it
-            auto score = [&](int i) {
-                const uint4 r = crec[i];
-                return (arow[r.x & 0xFFFFu] + __uint_as_float(r.y)) + (gs + brow[r.x >> 16]);      // as in fbw_combine
-            };
-            const int e0 = cb[d], e1 = cb[d + 1];
-            float smin = INF_F;
-            for (int i = e0; i < e1; i++) smin = fminf(smin, score(i));
-            if (!(smin < INF_F)) continue;                    // a hole: no edge of the slot is alive in this frame
-            float sum = 0.f;
-            for (int i = e0; i < e1; i++) sum += __builtin_amdgcn_exp2f(smin - score(i));
-            const double offs = a.offA[(size_t)b * a.T + t] + a.offB[(size_t)b * a.T + t];
-            const double loss = (double)a.sum_output[(size_t)t * a.B + b];
-            a.out[t * a.ost_t + b * a.ost_b + em] = (float)((((double)smin - (double)__builtin_amdgcn_logf(sum)) + offs) * (double)LN2 - loss);
+            float smin = INF_F, sum = 0.f;
+            if (few) {
+                float x[NE];
+#pragma unroll
+                for (int k = 0; k < NE; k++) { x[k] = (xa[tt][k] + __uint_as_float(r[k].y)) + (gs + xb[tt][k]); smin = fminf(smin, x[k]); }      // as in fbw_combine
+                if (!(smin < INF_F)) continue;                // a hole: no edge of the slot is alive in this frame
+#pragma unroll
+                for (int k = 0; k < NE; k++) sum += __builtin_amdgcn_exp2f(smin - x[k]);
+            } else {
+                const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
+                const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
+                auto score = [&](int i) {
+                    const uint4 q = crec[i];
+                    return (arow[q.x & 0xFFFFu] + __uint_as_float(q.y)) + (gs + brow[q.x >> 16]);
+                };
+                for (int i = e0; i < e1; i++) smin = fminf(smin, score(i));
+                if (!(smin < INF_F)) continue;
+                for (int i = e0; i < e1; i++) sum += __builtin_amdgcn_exp2f(smin - score(i));
+            }
+            a.out[t * a.ost_t + b * a.ost_b + em] = (float)(((double)smin - (double)__builtin_amdgcn_logf(sum)) * (double)LN2 + base[tt]);
         }
     }
 }
