@@ -1780,9 +1780,57 @@ __device__ __forceinline__ float slot_sum(const float* xs, const int c0, const i
     return s;
 }
 
+// The same in log space, for the -log output (NEGLOG instances of the kernels below): xs holds the raw
+// scores, +inf for a dead edge; the result is the smallest score m of the range and the sum of the
+// 2^(m - x) over it -- {+inf, 0} if no edge of the range is alive.  The reference adds a slot's edges in
+// log space too (fbw_op.cu:39-59,137-153) and so has a finite -log wherever some edge is alive, however
+// small its share of the frame; sums of probabilities relative to the frame minimum flush to zero from
+// 2^-126 of it and lose terms long before.
+struct LogSum { float mn, sum; };
+__device__ __forceinline__ LogSum slot_logsum(const float* xs, const int c0, const int c1) {
+    const int lane = threadIdx.x & 63;
+    const bool is_long = c1 - c0 > LONG_SLOT;
+    LogSum r = { INF_F, 0.f };
+    if (!is_long) {
+        for (int i = c0; i < c1; i++) r.mn = fminf(r.mn, xs[i]);
+        if (r.mn < INF_F)
+            for (int i = c0; i < c1; i++) r.sum += __builtin_amdgcn_exp2f(r.mn - xs[i]);
+    }
+    unsigned long long todo = __ballot(is_long);
+    while (todo) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int b0 = __builtin_amdgcn_readlane(c0, src), b1 = __builtin_amdgcn_readlane(c1, src);
+        float pm = INF_F;
+        for (int q = b0 + lane; q < b1; q += 64) pm = fminf(pm, xs[q]);
+        pm = lane63(wave_min_dpp(pm));
+        float p = 0.f;
+        if (pm < INF_F)
+            for (int q = b0 + lane; q < b1; q += 64) p += __builtin_amdgcn_exp2f(pm - xs[q]);
+        p = lane63(wave_sum_dpp(p));
+        if (lane == src) { r.mn = pm; r.sum = p; }
+    }
+    return r;
+}
+// a (+)= b for two pieces of one slot (edges staged in passes).  A slot that lies in one piece keeps the
+// bits of that piece.
+__device__ __forceinline__ void logsum_merge(LogSum& a, const LogSum b) {
+    if (!(b.mn < INF_F)) return;
+    if (!(a.mn < INF_F)) { a = b; return; }
+    const float m = fminf(a.mn, b.mn);
+    a.sum = a.sum * __builtin_amdgcn_exp2f(m - a.mn) + b.sum * __builtin_amdgcn_exp2f(m - b.mn);
+    a.mn = m;
+}
+// Element of the -log output from a slot's log-space sum {m, s}, the frame minimum mn and log2 of the frame
+// total (the sum of the 2^(mn - x) over all edges of the frame): -ln of s * 2^(mn - m) / total.
+__device__ __forceinline__ float neg_log_value(const LogSum s, const float mn, const float logtot) {
+    return s.mn < INF_F ? (((s.mn - mn) - __builtin_amdgcn_logf(s.sum)) + logtot) * LN2 : INF_F;
+}
+
 // (three waves per SIMD: with the headline workload's 48 KB row image three workgroups share a
 // compute unit, and the register count must not stand in the way)
-template <bool SYNC>
+// NEGLOG: the instance for the -log output (I6FBW_OUT_NEG_LOG), which sums a slot's edges in log space.
+template <bool SYNC, bool NEGLOG>
 __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
     __shared__ float redmin[COMB_THREADS / 64];
@@ -1851,7 +1899,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
                               a.offA + (size_t)b * T, a.offB + (size_t)b * T, a.out, a.ost_t, a.ost_b, a.sum_output, gred);
         return;
     }
-    const bool prob = a.out_mode != I6FBW_OUT_NEG_LOG;
+    constexpr bool prob = !NEGLOG;
     const float hole = prob ? 0.f : INF_F;
     const float psign = a.out_mode == I6FBW_OUT_NEG_PROB ? -1.f : 1.f;
 
@@ -1874,8 +1922,9 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     const float* bbase = a.beta + (size_t)T * soff;
     const float* gbase = a.gtab + (size_t)T * goff;
 
-    // writes the image positions of one frame from the per-slot sums, then streams the row out
-    auto finish_row = [&](int t, float mn, float tot, const float* sd, const int* em, int nslot_regs, double offs) {
+    // writes the image positions of one frame from the per-slot sums (sd: sums of probabilities relative to
+    // the frame minimum; NEGLOG: ls, the sums in log space), then streams the row out
+    auto finish_row = [&](int t, float mn, float tot, const float* sd, const LogSum* ls, const int* em, int nslot_regs, double offs) {
         const bool dead = mn == INF_F;
         const float logtot = __builtin_amdgcn_logf(tot);
         if (tid == 0)
@@ -1890,7 +1939,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             // their positions get the hole value back.
             auto value = [&](int js) -> float {
                 if (prob) return sd[js] * inv;
-                return (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+                return dead ? INF_F : neg_log_value(ls[js], mn, logtot);
             };
             float* base = orow - sh;
             const int W = a.tile_w, P = sh + F;
@@ -1927,7 +1976,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             if (d < D) {
                 float v;
                 if (prob) v = sd[js] * inv;
-                else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
+                else v = dead ? INF_F : neg_log_value(ls[js], mn, logtot);
                 image[sh + em[js]] = v;
             }
         }
@@ -1977,19 +2026,30 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             const double offs = voff;
             if (t + 1 < tv) fetch(t + 1);
             const float mn = block_min256(lmin, redmin);
+            // The frame normaliser (fbw_op.cu:115-134) is the sum of the probabilities relative to the frame
+            // minimum: of the per-emission sums, or, in the -log instance, which has no such sums, of the edges'
+            // in edge order per thread -- on every path of either dense writer edge i belongs to thread i mod 256,
+            // so each instance gives the same bits wherever it runs.
+            float part = 0.f;
 #pragma unroll
-            for (int j = 0; j < JE; j++) xs[tid + j * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
-            __syncthreads();
-            // per-emission sums in fixed (input) order, then the frame normaliser (fbw_op.cu:115-134)
+            for (int j = 0; j < JE; j++) {
+                const float p = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
+                if (NEGLOG) part += p;
+                xs[tid + j * COMB_THREADS] = NEGLOG ? x[j] : p;
+            }
+            float tot = 0.f;
+            if (NEGLOG) tot = block_sum256(part, redsum);     // (its barrier also publishes xs)
+            else __syncthreads();
+            // per-emission sums in fixed (input) order
             float sd[JS];
-            float lsum = 0.f;
+            LogSum ls[JS];
 #pragma unroll
             for (int js = 0; js < JS; js++) {
-                sd[js] = slot_sum(xs, c0[js], c1[js]);
-                lsum += sd[js];
+                if (NEGLOG) ls[js] = slot_logsum(xs, c0[js], c1[js]);
+                else { sd[js] = slot_sum(xs, c0[js], c1[js]); part += sd[js]; }
             }
-            const float tot = block_sum256(lsum, redsum);
-            finish_row(t, mn, tot, sd, em, JS, offs);
+            if (!NEGLOG) tot = block_sum256(part, redsum);
+            finish_row(t, mn, tot, sd, ls, em, JS, offs);
         }
     } else if (nE <= COMB_MID_EDGES && D <= COMB_MID_SLOTS) {
         // medium sequences: this thread's edges still stay in registers for the whole strip (sixteen
@@ -2026,31 +2086,38 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             const double offs = tid == 0 ? load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t) : 0.0;
             const float mn = block_min256(lmin, redmin);
             float sd[JS];
+            LogSum ls[JS];
 #pragma unroll
-            for (int js = 0; js < JS; js++) sd[js] = 0.f;
+            for (int js = 0; js < JS; js++) { sd[js] = 0.f; ls[js].mn = INF_F; ls[js].sum = 0.f; }
+            float part = 0.f;         // see the fast path
 #pragma unroll
             for (int p = 0; p < JE / JP; p++) {
                 if (p < npass) {
                     const int p0 = p * COMB_XS, p1 = min(nE, p0 + COMB_XS);
                     if (p > 0) __syncthreads();
 #pragma unroll
-                    for (int jj = 0; jj < JP; jj++)
-                        xs[tid + jj * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[p * JP + jj]);
+                    for (int jj = 0; jj < JP; jj++) {
+                        const float pr = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[p * JP + jj]);
+                        if (NEGLOG) part += pr;
+                        xs[tid + jj * COMB_THREADS] = NEGLOG ? x[p * JP + jj] : pr;
+                    }
                     __syncthreads();
 #pragma unroll
                     for (int js = 0; js < JS; js++) {
                         const int d = tid + js * COMB_THREADS;
                         int e0 = 0, e1 = 0;
                         if (d < D) { e0 = max(cb[d], p0) - p0; e1 = min(cb[d + 1], p1) - p0; }
-                        sd[js] += slot_sum(xs, e0, e1);
+                        if (NEGLOG) logsum_merge(ls[js], slot_logsum(xs, e0, e1));
+                        else sd[js] += slot_sum(xs, e0, e1);
                     }
                 }
             }
-            float lsum = 0.f;
+            if (!NEGLOG) {
 #pragma unroll
-            for (int js = 0; js < JS; js++) lsum += sd[js];
-            const float tot = block_sum256(lsum, redsum);
-            finish_row(t, mn, tot, sd, em, JS, offs);
+                for (int js = 0; js < JS; js++) part += sd[js];
+            }
+            const float tot = block_sum256(part, redsum);
+            finish_row(t, mn, tot, sd, ls, em, JS, offs);
         }
     } else {
         // general path: edge records re-read per frame, edges staged through LDS in passes of
@@ -2067,133 +2134,38 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             for (int i = tid; i < nE; i += COMB_THREADS) lmin = fminf(lmin, score(i));
             const float mn = block_min256(lmin, redmin);
             float sd[COMB_JD];
+            LogSum ls[COMB_JD];
             int em[COMB_JD];
 #pragma unroll
-            for (int jd = 0; jd < COMB_JD; jd++) { sd[jd] = 0.f; em[jd] = 0; }
+            for (int jd = 0; jd < COMB_JD; jd++) { sd[jd] = 0.f; ls[jd].mn = INF_F; ls[jd].sum = 0.f; em[jd] = 0; }
+            float part = 0.f;         // see the fast path
             for (int p0 = 0; p0 < nE; p0 += COMB_XS) {
                 const int p1 = min(nE, p0 + COMB_XS);
                 __syncthreads();
-                for (int i = p0 + tid; i < p1; i += COMB_THREADS)
-                    xs[i - p0] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - score(i));
+                for (int i = p0 + tid; i < p1; i += COMB_THREADS) {
+                    const float x = score(i);
+                    const float pr = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x);
+                    if (NEGLOG) part += pr;
+                    xs[i - p0] = NEGLOG ? x : pr;
+                }
                 __syncthreads();
 #pragma unroll
                 for (int jd = 0; jd < COMB_JD; jd++) {
                     const int d = tid + jd * COMB_THREADS;
                     int e0 = 0, e1 = 0;
                     if (d < D) { e0 = max(cb[d], p0) - p0; e1 = min(cb[d + 1], p1) - p0; }
-                    sd[jd] += slot_sum(xs, e0, e1);
+                    if (NEGLOG) logsum_merge(ls[jd], slot_logsum(xs, e0, e1));
+                    else sd[jd] += slot_sum(xs, e0, e1);
                 }
             }
-            float lsum = 0.f;
 #pragma unroll
             for (int jd = 0; jd < COMB_JD; jd++) {
                 const int d = tid + jd * COMB_THREADS;
                 if (d < D) em[jd] = de[d];
-                lsum += sd[jd];
+                if (!NEGLOG) part += sd[jd];
             }
-            const float tot = block_sum256(lsum, redsum);
-            finish_row(t, mn, tot, sd, em, COMB_JD, load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t));
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------------------------
-// -log output only: posteriors below float's range.  The kernels above sum a slot's probabilities
-// relative to the frame minimum; a slot whose share is below 2^-126 of that flushes to zero and its
-// element comes out as +inf, while the reference, which adds in log space (fbw_op.cu:115-134), has
-// a finite value there (a -log above 87).  This pass goes over the elements of the emissions a
-// sequence uses, frame by frame, after the dense write: where one holds +inf although an edge of its
-// slot is alive -- or a value so large that its sum may have lost terms --, the slot is summed once more relative
-// to its own minimum,
-//     -log p = ln 2 * (min_e x_e - log2 sum_e 2^(min - x_e) + row offsets) - loss,
-// with the frame's loss as the dense write left it.  A pass of its own, because the same lines
-// inside fbw_flat cost that kernel its register budget (and the dense write half its speed).  Sequences
-// on the general path add in log space anyway.  About as much traffic as the gather, in this output
-// mode only.
-// ---------------------------------------------------------------------------------------------
-constexpr int TAIL_FRAMES = 8;
-// (the emission scores from am_scores themselves, as the gather scales them: by now the compact table may hold the flat
-// writer's values)
-// cp: the flat writer's compact values [seq][t][slot] (what it copied into the tensor; read in place of the tensor's
-// scattered elements for the sequences it wrote), or null.
-__global__ __launch_bounds__(COMB_THREADS) void fbw_neg_log_tail(CombArgs a, const float* am, long long st_t, long long st_b, float scale,
-                                                                 const float* cp) {
-    const int b = blockIdx.y, t0 = blockIdx.x * TAIL_FRAMES, tid = threadIdx.x;
-    const SeqMeta m = a.meta[b];
-    if (rec_class(m) <= 0) return;
-    const int nt = min(m.L, t0 + TAIL_FRAMES) - t0;
-    if (nt <= 0) return;
-    const int D = m.D, SP = m.SP, DP = m.DP;
-    const long long soff = state_off(m.edge_begin, b), goff = slot_off(m.edge_begin, b);
-    const uint4* crec = a.crec + m.edge_begin;
-    const int* cb = a.cbegin + goff;
-    const int* de = a.demis + goff;
-    const float* compact = (cp && flat_fast(m)) ? cp + (size_t)a.T * goff : nullptr;
-    for (int d = tid; d < D; d += COMB_THREADS) {
-        const int em = de[d];
-        // the values of all frames first: the loads are in flight together
-        float v[TAIL_FRAMES], g[TAIL_FRAMES];       // and the slot's emission score in each of them (all edges of a slot share it)
-        double base[TAIL_FRAMES];                   // row offsets * ln 2 - loss of the frame
-#pragma unroll
-        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            v[tt] = 0.f; g[tt] = INF_F; base[tt] = 0.0;
-            if (tt < nt) {
-                base[tt] = (a.offA[(size_t)b * a.T + t0 + tt] + a.offB[(size_t)b * a.T + t0 + tt]) * (double)LN2
-                           - (double)a.sum_output[(size_t)(t0 + tt) * a.B + b];
-                v[tt] = compact ? compact[(size_t)(t0 + tt) * DP + d] : a.out[(t0 + tt) * a.ost_t + b * a.ost_b + em];
-                g[tt] = __builtin_nontemporal_load(&am[(long long)(t0 + tt) * st_t + (long long)b * st_b + em]);
-            }
-        }
-        // (not only +inf: from 2^-100 of the frame minimum down a sum may have lost some of its terms; as a -log
-        // that is 69 and more, whatever the frame's normaliser, which is at least 1)
-        bool any = false;
-#pragma unroll
-        for (int tt = 0; tt < TAIL_FRAMES; tt++) any |= v[tt] > 69.f;
-        if (!any) continue;
-        const int e0 = cb[d], e1 = cb[d + 1];
-        constexpr int NE = 4;                 // edges of a slot held in registers (the usual slot has one or two)
-        uint4 r[NE];
-#pragma unroll
-        for (int k = 0; k < NE; k++) r[k] = e0 + k < e1 ? crec[e0 + k] : make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);      // weight +inf: contributes nothing
-        const bool few = e1 - e0 <= NE;
-        // the row elements of all frames and edges first (in flight together), then the arithmetic
-        float xa[TAIL_FRAMES][NE], xb[TAIL_FRAMES][NE];
-#pragma unroll
-        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            const int t = t0 + tt;
-            const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
-            const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
-#pragma unroll
-            for (int k = 0; k < NE; k++) {
-                xa[tt][k] = INF_F; xb[tt][k] = INF_F;
-                if (few && v[tt] > 69.f && e0 + k < e1) { xa[tt][k] = arow[r[k].x & 0xFFFFu]; xb[tt][k] = brow[r[k].x >> 16]; }
-            }
-        }
-#pragma unroll
-        for (int tt = 0; tt < TAIL_FRAMES; tt++) {
-            if (!(v[tt] > 69.f)) continue;
-            const int t = t0 + tt;
-            const float gs = g[tt] == INF_F ? INF_F : g[tt] * scale;          // as fbw_gather scales it
-            float smin = INF_F, sum = 0.f;
-            if (few) {
-                float x[NE];
-#pragma unroll
-                for (int k = 0; k < NE; k++) { x[k] = (xa[tt][k] + __uint_as_float(r[k].y)) + (gs + xb[tt][k]); smin = fminf(smin, x[k]); }      // as in fbw_combine
-                if (!(smin < INF_F)) continue;                // a hole: no edge of the slot is alive in this frame
-#pragma unroll
-                for (int k = 0; k < NE; k++) sum += __builtin_amdgcn_exp2f(smin - x[k]);
-            } else {
-                const float* arow = a.alpha + (size_t)a.T * soff + (size_t)t * SP;
-                const float* brow = a.beta + (size_t)a.T * soff + (size_t)t * SP;
-                auto score = [&](int i) {
-                    const uint4 q = crec[i];
-                    return (arow[q.x & 0xFFFFu] + __uint_as_float(q.y)) + (gs + brow[q.x >> 16]);
-                };
-                for (int i = e0; i < e1; i++) smin = fminf(smin, score(i));
-                if (!(smin < INF_F)) continue;
-                for (int i = e0; i < e1; i++) sum += __builtin_amdgcn_exp2f(smin - score(i));
-            }
-            a.out[t * a.ost_t + b * a.ost_b + em] = (float)(((double)smin - (double)__builtin_amdgcn_logf(sum)) * (double)LN2 + base[tt]);
+            const float tot = block_sum256(part, redsum);
+            finish_row(t, mn, tot, sd, ls, em, COMB_JD, load_x<SYNC>(offA + t) + load_x<SYNC>(offB + t));
         }
     }
 }
@@ -2270,7 +2242,7 @@ __device__ __forceinline__ int middle_out(const int i, const int n, const int mi
     return up > down ? mid + (i - down) : mid - (i - up);
 }
 
-template <bool SYNC>
+template <bool SYNC, bool NEGLOG>
 __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const int t0, float* xs, float* redmin, float* redsum,
                                           int* s_ok) {
     const CombArgs& a = fa.c;
@@ -2309,7 +2281,10 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
             return;
         }
     }
-    const bool prob = a.out_mode != I6FBW_OUT_NEG_LOG;
+    // (A run-time value in the instance for the posterior modes, although the host launches the NEGLOG instance for the
+    // -log output: with the branch folded away the compiler arranges the rest so that it needs five registers more
+    // than the 64 this kernel is launched for, and spills them inside the frame loop.)
+    const bool prob = NEGLOG ? false : a.out_mode != I6FBW_OUT_NEG_LOG;
     const float psign = a.out_mode == I6FBW_OUT_NEG_PROB ? -1.f : 1.f;
     const int nE = m.n_edges, D = m.D, SP = m.SP, DP = m.DP;
     const long long soff = state_off(m.edge_begin, b), goff = slot_off(m.edge_begin, b);
@@ -2383,16 +2358,26 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
             const float lmin = lmins[f];
             const double offs = voffs[f];
             const float mn = block_min256(lmin, redmin);
-            for (int i = tid; i < nE; i += COMB_THREADS) xs[i] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - xs[i]);    // (each thread its own)
-            __syncthreads();
             float sd[JSL];
-            float lsum = 0.f;
+            LogSum ls[JSL];
+            float tot;
+            if (NEGLOG) {
+                float part = 0.f;         // the frame normaliser, as in fbw_combine
+                for (int i = tid; i < nE; i += COMB_THREADS) part += mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - xs[i]);
+                tot = block_sum256(part, redsum);
 #pragma unroll
-            for (int js = 0; js < JSL; js++) {
-                sd[js] = slot_sum(xs, (int)(crl[js] & 0xFFFFu), (int)(crl[js] >> 16));
-                lsum += sd[js];
+                for (int js = 0; js < JSL; js++) ls[js] = slot_logsum(xs, (int)(crl[js] & 0xFFFFu), (int)(crl[js] >> 16));
+            } else {
+                for (int i = tid; i < nE; i += COMB_THREADS) xs[i] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - xs[i]);    // (each thread its own)
+                __syncthreads();
+                float lsum = 0.f;
+#pragma unroll
+                for (int js = 0; js < JSL; js++) {
+                    sd[js] = slot_sum(xs, (int)(crl[js] & 0xFFFFu), (int)(crl[js] >> 16));
+                    lsum += sd[js];
+                }
+                tot = block_sum256(lsum, redsum);
             }
-            const float tot = block_sum256(lsum, redsum);
             const bool dead = mn == INF_F;
             const float logtot = __builtin_amdgcn_logf(tot);
             if (tid == 0)
@@ -2405,6 +2390,7 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
                 if (d < D) {
                     float v;
                     if (prob) v = sd[js] * inv;
+                    else if (NEGLOG) v = dead ? INF_F : neg_log_value(ls[js], mn, logtot);
                     else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
                     store_agent(cprow + d, v);
                 }
@@ -2455,18 +2441,34 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
         const double offs = voff;
         if (t + 1 < tv) fetch(t + 1);
         const float mn = block_min256(lmin, redmin);
-#pragma unroll
-        for (int j = 0; j < JE; j++) xs[tid + j * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
-        __syncthreads();
-        // per-emission sums in fixed (input) order, then the frame normaliser (fbw_op.cu:115-134)
+        // the frame normaliser (fbw_op.cu:115-134), as in fbw_combine
         float sd[JS];
-        float lsum = 0.f;
+        LogSum ls[JS];
+        float tot;
+        if (NEGLOG) {
+            float part = 0.f;
 #pragma unroll
-        for (int js = 0; js < JS; js++) {
-            sd[js] = slot_sum(xs, (int)(cr[js] & 0xFFFFu), (int)(cr[js] >> 16));
-            lsum += sd[js];
+            for (int j = 0; j < JE; j++) {
+                part += mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
+                xs[tid + j * COMB_THREADS] = x[j];
+            }
+            tot = block_sum256(part, redsum);      // (its barrier also publishes xs)
+            // per-emission sums in fixed (input) order
+#pragma unroll
+            for (int js = 0; js < JS; js++) ls[js] = slot_logsum(xs, (int)(cr[js] & 0xFFFFu), (int)(cr[js] >> 16));
+        } else {
+#pragma unroll
+            for (int j = 0; j < JE; j++) xs[tid + j * COMB_THREADS] = mn == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn - x[j]);
+            __syncthreads();
+            // per-emission sums in fixed (input) order
+            float lsum = 0.f;
+#pragma unroll
+            for (int js = 0; js < JS; js++) {
+                sd[js] = slot_sum(xs, (int)(cr[js] & 0xFFFFu), (int)(cr[js] >> 16));
+                lsum += sd[js];
+            }
+            tot = block_sum256(lsum, redsum);
         }
-        const float tot = block_sum256(lsum, redsum);
         const bool dead = mn == INF_F;
         const float logtot = __builtin_amdgcn_logf(tot);
         if (tid == 0)
@@ -2479,6 +2481,7 @@ __device__ __forceinline__ void flat_post(const FlatArgs& fa, const int b, const
             if (d < D) {
                 float v;
                 if (prob) v = sd[js] * inv;
+                else if (NEGLOG) v = dead ? INF_F : neg_log_value(ls[js], mn, logtot);
                 else v = (dead || sd[js] == 0.f) ? INF_F : (logtot - __builtin_amdgcn_logf(sd[js])) * LN2;
                 store_agent(cprow + d, v);
             }
@@ -2698,8 +2701,9 @@ __device__ __forceinline__ void flat_write(const FlatArgs& fa, const long long r
 #endif
 }
 
-template <bool SYNC>
-__global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs fa) {
+// (the -log instance needs a few registers more for its sums in log space: six workgroups per compute unit)
+template <bool SYNC, bool NEGLOG>
+__global__ __launch_bounds__(COMB_THREADS, NEGLOG ? (I6_FLAT_OCC < 6 ? I6_FLAT_OCC : 6) : I6_FLAT_OCC) void fbw_flat(FlatArgs fa) {
     // image of a write job; staging area of a posterior job (the scores of the edges of its frames)
     __shared__ float4a img4[FLAT_TCF * FLAT_EDGES / 4];
     static_assert(FLAT_TCF * FLAT_EDGES >= FLAT_W, "the image fits");
@@ -2732,7 +2736,7 @@ __global__ __launch_bounds__(COMB_THREADS, I6_FLAT_OCC) void fbw_flat(FlatArgs f
     const int Lmid = fa.layout == 0 ? fa.c.sync[6] : fa.c.meta[b].L;
     const int strip = middle_out(i, n, min(n - 1, (Lmid / 2) / TC));
     if (job < 0) {
-        flat_post<SYNC>(fa, b, strip * TC + qf * FLAT_TCF, (float*)img4, redmin, redsum, s_kind);
+        flat_post<SYNC, NEGLOG>(fa, b, strip * TC + qf * FLAT_TCF, (float*)img4, redmin, redsum, s_kind);
         return;
     }
     const long long row0 = fa.layout == 0 ? (long long)strip * TC * B : (long long)b * T + strip * TC;
@@ -2844,6 +2848,18 @@ void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
     else hipLaunchKernelGGL(fbw_prepare<1024>, dim3(3, pa.B), dim3(1024), lds, s, pa);
 }
 
+// The dense writers, in the instance for the output mode (NEGLOG: the -log output, summed in log space)
+template <bool SYNC>
+void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStream_t s, const CombArgs& ca) {
+    if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true>), grid, dim3(COMB_THREADS), lds, s, ca);
+    else hipLaunchKernelGGL((fbw_combine<SYNC, false>), grid, dim3(COMB_THREADS), lds, s, ca);
+}
+template <bool SYNC>
+void launch_flat(const bool neglog, const dim3 grid, hipStream_t s, const FlatArgs& fa) {
+    if (neglog) hipLaunchKernelGGL((fbw_flat<SYNC, true>), grid, dim3(COMB_THREADS), 0, s, fa);
+    else hipLaunchKernelGGL((fbw_flat<SYNC, false>), grid, dim3(COMB_THREADS), 0, s, fa);
+}
+
 // Device facts and kernel attributes; creates nothing (i6fbw_run_static stops here).
 int device_init(Pipeline& p) {
     if (p.attr_ready) return I6FBW_OK;
@@ -2854,10 +2870,10 @@ int device_init(Pipeline& p) {
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_combine<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+    for (const void* k : {(const void*)fbw_combine<true, false>, (const void*)fbw_combine<false, false>,
+                          (const void*)fbw_combine<true, true>, (const void*)fbw_combine<false, true>})
+        HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     hipFuncAttributes attr;
-    HIP_TRY(hipFuncSetAttribute((const void*)fbw_flat<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 0));
     HIP_TRY(hipFuncGetAttributes(&attr, (const void*)fbw_recurse_dense<true>));
     p.dense_regs = attr.numRegs;
     // address of the current device's copy of the built-in workspace
@@ -3132,6 +3148,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
 
     const dim3 g_grid((unsigned)B * ((T + TG - 1) / TG)), c_grid((unsigned)B * ((T + TC - 1) / TC));
     const dim3 p_grid(B, (T + TC - 1) / TC);
+    const bool neglog = out_mode == I6FBW_OUT_NEG_LOG;      // the dense write then sums in log space (its NEGLOG instances)
     if ((long long)B * ((T + TG - 1) / TG) > 0x7fffffffLL) return I6FBW_ERR_INVALID_ARGUMENT;
     PrepArgs pa;
     pa.edges = edges; pa.edge_stride = edge_row_stride; pa.weights = weights;
@@ -3162,7 +3179,6 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     ca.out = out; ca.sum_output = sum_output; ca.ost_t = out_stride_t; ca.ost_b = out_stride_b; ca.sync = sync;
     ca.tile_w = tiled ? COMB_TILE_W : 0;
     ca.direct_only = 0;
-    const dim3 tail_grid((unsigned)((T + TAIL_FRAMES - 1) / TAIL_FRAMES), (unsigned)B);
     // The dense tensor goes out in flat spans (fbw_flat) if it is one contiguous block in either
     // order of frames and sequences, rows are long enough for a span to cut at most two of them,
     // and the tensor is large (for small problems the row writer is as good).
@@ -3270,14 +3286,10 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         HIP_TRY(hipGetLastError());
         if (flat) {
             // (the row kernel first: it only has the sequences that are too large for the other one)
-            { StageTimer tm(4, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
-            { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_flat<false>, dim3((unsigned)flat_grid), dim3(COMB_THREADS), 0, s, fa); }
-        } else { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<false>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+            { StageTimer tm(4, s, timed); launch_combine<false>(neglog, c_grid, comb_lds, s, ca); }
+            { StageTimer tm(3, s, timed); launch_flat<false>(neglog, dim3((unsigned)flat_grid), s, fa); }
+        } else { StageTimer tm(3, s, timed); launch_combine<false>(neglog, c_grid, comb_lds, s, ca); }
         HIP_TRY(hipGetLastError());
-        if (out_mode == I6FBW_OUT_NEG_LOG) {
-            hipLaunchKernelGGL(fbw_neg_log_tail, tail_grid, dim3(COMB_THREADS), 0, s, ca, ga.am, ga.st_t, ga.st_b, ga.scale, flat ? (const float*)fa.cp : (const float*)nullptr);
-            HIP_TRY(hipGetLastError());
-        }
         return I6FBW_OK;
     }
 
@@ -3300,7 +3312,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         // register file).  It has nothing to do for the usual batch.
         HIP_TRY(hipEventRecord(P.gathered, s));
         HIP_TRY(hipStreamWaitEvent(sP, P.gathered, 0));
-        { StageTimer tm(4, sP, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, sP, ca); }
+        { StageTimer tm(4, sP, timed); launch_combine<true>(neglog, c_grid, comb_lds, sP, ca); }
         HIP_TRY(hipGetLastError());
         HIP_TRY(hipEventRecord(P.doneP, sP));
     }
@@ -3311,17 +3323,13 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
 #ifdef I6_TRACE
     if (getenv("I6FBW_DBG_SERIAL_COMBINE")) HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
 #endif
-    if (flat) { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_flat<true>, dim3((unsigned)flat_grid), dim3(COMB_THREADS), 0, s, fa); }
-    else { StageTimer tm(3, s, timed); hipLaunchKernelGGL(fbw_combine<true>, c_grid, dim3(COMB_THREADS), comb_lds, s, ca); }
+    if (flat) { StageTimer tm(3, s, timed); launch_flat<true>(neglog, dim3((unsigned)flat_grid), s, fa); }
+    else { StageTimer tm(3, s, timed); launch_combine<true>(neglog, c_grid, comb_lds, s, ca); }
     HIP_TRY(hipGetLastError());
     // join: both finish well before the dense write does
     HIP_TRY(hipStreamWaitEvent(s, P.doneP, 0));
     HIP_TRY(hipStreamWaitEvent(s, P.doneR, 0));
     join_guard.joined = true;
-    if (out_mode == I6FBW_OUT_NEG_LOG) {
-        hipLaunchKernelGGL(fbw_neg_log_tail, tail_grid, dim3(COMB_THREADS), 0, s, ca, ga.am, ga.st_t, ga.st_b, ga.scale, flat ? (const float*)fa.cp : (const float*)nullptr);
-        HIP_TRY(hipGetLastError());
-    }
     return I6FBW_OK;
 }
 }  // namespace

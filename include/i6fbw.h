@@ -40,10 +40,9 @@ enum {
 /* Layout of the posterior tensor written by i6fbw_run. */
 enum {
     I6FBW_OUT_NEG_LOG = 0,   /* -log posterior, +inf where nothing contributes: what fbw_core.fbw returns
-                                (fbw_op.cu:366-377,392); finite wherever some edge contributes, however little (the
-                                reference adds in log space: a pass of its own after the dense write takes the
-                                elements above 69, whose sums of probabilities may have left float's range, once
-                                more in log space; it costs this mode about as much again as the rest of the call) */
+                                (fbw_op.cu:366-377,392); finite wherever some edge contributes, however little: the
+                                dense write of this mode adds the edges of an emission in log space, as the
+                                reference does (fbw_op.cu:39-59,137-153) */
     I6FBW_OUT_PROB = 1,      /* posterior itself, 0 where nothing contributes: what
                                 FastBaumWelchLoss.backward derives from it (fbw/__init__.py:40-44) */
     I6FBW_OUT_NEG_PROB = 2   /* minus the posterior: the gradient that reaches `log_probs` in fbw_loss

@@ -130,7 +130,10 @@ def test_kernels_stay_within_their_register_budgets():
         return found
 
     for name, r in kernels("fbw_flat").items():
-        assert r["scratch"] == 0 and r["vgprs"] <= 64 and r["occupancy"] == 8, (name, r)
+        if name.endswith("Lb1EEEvNS_8FlatArgsE"):      # the instance for the -log output: sums in log space, six waves per SIMD
+            assert r["scratch"] == 0 and r["vgprs"] <= 80 and r["occupancy"] >= 6, (name, r)
+        else:
+            assert r["scratch"] == 0 and r["vgprs"] <= 64 and r["occupancy"] == 8, (name, r)
     for fragment in ("fbw_gather", "fbw_prepare", "fbw_padfill", "fbw_scan_sorted", "11fbw_recurseI", "vit_align"):
         for name, r in kernels(fragment).items():
             assert r["scratch"] == 0, (name, r)

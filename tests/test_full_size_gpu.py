@@ -62,6 +62,39 @@ def test_full_size(oracle, name):
     assert float((post2 - post).abs().max()) <= 1e-4
 
 
+@pytest.mark.parametrize("name", ["cart", "ctc"])
+def test_full_size_neg_log(oracle, name):
+    """The -log output (what fbw_core.fbw returns, fbw_op.cu:366-377,392) at full size: the values themselves in the log
+    domain, and +inf in exactly the oracle's places -- the reference adds in log space (fbw_op.cu:39-59,137-153) and has
+    a finite -log wherever some edge is alive, far below the range of a float posterior."""
+    W = make_workload(name)
+    print(f"full size -log {name}: T={W.T} B={W.B} F={W.F} E={W.E}", flush=True)
+    P = DeviceProblem(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states)
+    out, loss = P.run(cabi.OUT_NEG_LOG)
+    torch.cuda.synchronize()
+    out, loss = out.clone(), loss.clone()          # (the problem's buffers are written again below)
+    want_out, want_loss = oracle.fbw_oracle(W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens,
+                                            W.n_states, threads=min(16, W.B))
+    np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
+    got = out.cpu().numpy()
+    atol = 2e-3 + 1.2e-7 * float(np.abs(want_loss).max())      # a large -log is the difference of two numbers of the size of the loss
+    n_fin = n_deep = 0
+    for t0 in range(0, W.T, 100):
+        g, w = got[t0:t0 + 100], want_out[t0:t0 + 100]
+        fin = np.isfinite(w)
+        assert (np.isposinf(g) == ~fin).all(), t0
+        np.testing.assert_allclose(g[fin], w[fin], rtol=2e-5, atol=atol)
+        n_fin += int(fin.sum())
+        n_deep += int((w[fin] > 88.0).sum())
+    print(f"full size -log {name}: {n_fin} finite elements, {n_deep} of them beyond the range of a float posterior", flush=True)
+    assert n_deep > 0       # the case the log-space sums are there for
+    # the posterior mode on the same inputs: same loss to rounding, exp(-out) = posterior
+    post, loss1 = P.run(cabi.OUT_PROB)
+    torch.cuda.synchronize()
+    assert torch.all((loss1 - loss).abs() <= 1e-6 * loss.abs())
+    assert float((torch.exp(-out) - post).abs().max()) <= 2e-6
+
+
 def test_full_size_best_path(oracle):
     """Best path on the headline automata: bit-identical to the oracle, and the path's own score,
     re-accumulated in float64 along the alignment, matches the reported score."""

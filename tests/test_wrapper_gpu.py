@@ -71,8 +71,8 @@ def test_core_fbw_contract(oracle):
     assert out.shape == (W.T, W.B, W.F) and loss.shape == (W.T, W.B)
     np.testing.assert_allclose(loss.cpu().numpy(), want_loss, rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(posterior(out.cpu().numpy()), posterior(want_out), atol=1e-4)
-    tiny = posterior(want_out) < 1e-30      # a posterior below float range may be a hole on one side only
-    assert ((np.isposinf(out.cpu().numpy()) | tiny) == (np.isposinf(want_out) | tiny)).all()
+    # holes in exactly the same places, also where a posterior is below float's range: both sides add in log space
+    assert (np.isposinf(out.cpu().numpy()) == np.isposinf(want_out)).all()
     # the autograd path yields the same numbers
     from i6_native_ops_amd.fbw import FastBaumWelchLoss
     am = torch.from_numpy(W.am_scores).to(dev).requires_grad_(True)
