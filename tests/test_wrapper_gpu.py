@@ -80,7 +80,8 @@ def test_core_fbw_contract(oracle):
            torch.from_numpy(W.start_end_states).to(dev))
     l2 = FastBaumWelchLoss.apply(am, fsa, torch.from_numpy(W.seq_lens).to(dev))
     l2.sum().backward()
-    assert torch.equal(l2, loss)
+    # (the posterior mode behind the autograd path adds up the frame normaliser per emission, the -log mode per edge)
+    assert torch.all((l2 - loss).abs() <= 1e-6 * loss.abs())
     np.testing.assert_allclose(am.grad.cpu().numpy(), posterior(want_out), atol=1e-4)
 
 
