@@ -1,0 +1,1 @@
+from ._version import __version__  # noqa: F401

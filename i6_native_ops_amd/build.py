@@ -42,6 +42,18 @@ def kernel_resources(remarks):
     return out
 
 
+def sources_digest():
+    """sha256 over the device sources and the compiler flags: kept inside kernel_resources.json, so that a record
+    made from other sources than the ones present is recognised as such"""
+    import hashlib
+    h = hashlib.sha256(" ".join(HIP_FLAGS).encode())
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".inc", ".h")):
+            h.update(name.encode())
+            h.update(open(os.path.join(CSRC, name), "rb").read())
+    return h.hexdigest()
+
+
 def build_lib(out_root=PKG):
     """libi6fbw.so into <out_root>/fbw (out_root: this package in the source tree, or its copy in a build tree),
     and beside it kernel_resources.json: registers, scratch and occupancy of every kernel as the compiler reports
@@ -61,8 +73,10 @@ def build_lib(out_root=PKG):
         print("\n".join(other), flush=True)
     if done.returncode != 0:
         raise subprocess.CalledProcessError(done.returncode, cmd)
+    record = kernel_resources(remarks)
+    record["_sources_sha256"] = sources_digest()
     with open(os.path.join(out_root, "fbw", "kernel_resources.json"), "w") as f:
-        json.dump(kernel_resources(remarks), f, indent=1, sort_keys=True)
+        json.dump(record, f, indent=1, sort_keys=True)
     return lib
 
 

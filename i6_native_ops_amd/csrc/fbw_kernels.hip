@@ -1393,9 +1393,19 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     const long long goff = slot_off(m.edge_begin, b);
     const float* G = a.gtab + (size_t)T * goff;
     const int nsteps = L - 1;
-    const int npiece = DP >> 1;                       // DP is a multiple of 16
-    // my pieces of a row: lane + jl*64, clamped to the row
-    auto cc = [&](int jl) { return min(lane + jl * 64, npiece - 1); };
+    // My pieces of a row, lane + jl*64, come through buffer loads: the resource describes the one row (its address, its
+    // length in bytes), the lane's offset 8 * lane + 512 * jl is checked against that length by the hardware, and a piece
+    // past the end of the row comes back as zero without touching memory (it lands in LDS cells no edge refers to).
+    // One vector register addresses all pieces of all rows, where global loads clamped to the row took a 64-bit address
+    // per piece (with 32 pieces per lane those alone filled half of the register budget of the largest instance, which
+    // spilled); reading on past the row's end instead costs the large-automaton instance 3 % (its rows are read
+    // from the memory side while the gather is still writing).
+    const int lane8 = lane * 8;
+    auto piece = [&](const u64* row, int jl) -> u64 {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)row, 0, DP * 4, 0x00020000);
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(rs, lane8 + jl * 512, 0, SYNC ? 16 : 0);      // (16: sc1, the agent-scope load of load_agent)
+        return ((u64)v[1] << 32) | v[0];
+    };
     int* abort_flag = a.sync;
     const int* gflag = a.sync + SYNC_HDR + 2 * a.B + (size_t)b * ((T + TG - 1) / TG);
     const int nstrip = (L + TG - 1) / TG;
@@ -1421,12 +1431,12 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
     if (nsteps > 0) {
         const u64* r0 = rowp(0);
 #pragma unroll
-        for (int jl = 0; jl < JL; jl++) ((u64*)am0)[lane + jl * 64] = load_x<SYNC>(r0 + cc(jl));
+        for (int jl = 0; jl < JL; jl++) ((u64*)am0)[lane + jl * 64] = piece(r0, jl);
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const u64* rp = rowp(1 + p);
 #pragma unroll
-            for (int jl = 0; jl < JL; jl++) g[p][jl] = load_x<SYNC>(rp + cc(jl));
+            for (int jl = 0; jl < JL; jl++) g[p][jl] = piece(rp, jl);
         }
     }
     lds_barrier();      // pairs with the barrier at the end of recurse_init
@@ -1439,7 +1449,7 @@ __device__ __forceinline__ void recurse_load(const RecArgs& a, const SeqMeta& m,
 #pragma unroll
             for (int jl = 0; jl < JL; jl++) {
                 amn[lane + jl * 64] = g[q][jl];
-                g[q][jl] = load_x<SYNC>(nxt + cc(jl));
+                g[q][jl] = piece(nxt, jl);
             }
 #ifdef I6_TRACE
             { const int i_ = i0 + q; const bool tr_ = blockIdx.x == 0 && i_ >= 400 && i_ < 432 && lane == 0;
@@ -1585,8 +1595,11 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     const bool small_tight = cls == 1 && m.SP <= 256 && m.L < 4LL * m.S;
     const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES);
     // (there double costs half of the recursion time again, so only from 384 frames on, where the
-    // rounding of float has had time to add up; but for every sequence with one state per thread)
-    if (DENSE && cls == 1 && m.L >= 384 && (dir ? m.Kout : m.Kin) <= KMAX) {
+    // rounding of float has had time to add up -- but then for every sequence with one state per thread --
+    // and from 256 frames on for the tightly aligned ones: 140 monophone automata of 250-400 states over
+    // 320-400 frames came out at 8.7e-5 in float, 3.6e-5 in double; CTC automata of 40-120 states over 150-200
+    // frames are at 1.7e-5 in float and would pay 14 us per call)
+    if (DENSE && cls == 1 && (m.L >= 384 || (m.L >= 256 && 5LL * m.S > 3LL * m.L)) && (dir ? m.Kout : m.Kin) <= KMAX) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true, false>(a, m, b, dir, cls, st0, st0 + (T_ + 16), amr[0], amr[1], wmin);
     } else if (DENSE && cls >= 2 && (5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES)) {
@@ -1625,8 +1638,11 @@ __global__ __launch_bounds__(REC_BLOCK) void fbw_recurse(RecArgs a) {
 // The dense instance takes its LDS as dynamic shared memory (REC_LDS_FLOATS_F32 floats): with the
 // size known at compile time the compiler sees that at most two workgroups fit on a unit anyway
 // and ignores the register cap, and two workgroups then fill the register file.
+// (The cap of 96 registers is for the schedule in which gather and dense write run beside this kernel and need room on
+// its compute units; stage after stage -- the schedule the library chooses for such batches -- two workgroups have the
+// register file to themselves, four waves per SIMD with 128 registers each, and nothing spills inside the time loops.)
 template <bool SYNC>
-__global__ __launch_bounds__(REC_BLOCK_DENSE, 5) void fbw_recurse_dense(RecArgs a) {
+__global__ __launch_bounds__(REC_BLOCK_DENSE, SYNC ? 5 : 4) void fbw_recurse_dense(RecArgs a) {
     extern __shared__ __attribute__((aligned(16))) float dyn_lds[];
     recurse_workgroup<SYNC, 1>(a, dyn_lds);
 }
@@ -1830,6 +1846,9 @@ __device__ __forceinline__ float neg_log_value(const LogSum s, const float mn, c
 // (three waves per SIMD: with the headline workload's 48 KB row image three workgroups share a
 // compute unit, and the register count must not stand in the way)
 // NEGLOG: the instance for the -log output (I6FBW_OUT_NEG_LOG), which sums a slot's edges in log space.
+// (At three waves per SIMD the -log instance keeps a few values of its paths for sequences of more than 1024 edges
+// in scratch memory -- six reloads per frame there, none on the path for smaller sequences; at two it needs none, and
+// the monophone configuration, all of whose sequences are small, takes 8 % longer per call.)
 template <bool SYNC, bool NEGLOG>
 __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
@@ -3437,6 +3456,13 @@ const char* i6fbw_strerror(int code) {
 
 int i6fbw_set_spin_limit(int polls) {
     const int v = polls > 0 ? polls : SPIN_LIMIT;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return I6FBW_ERR_INVALID_ARGUMENT;
+    // no call of the library is being enqueued on this device while the limit changes, and none that was enqueued
+    // before is still running: a kernel sees one limit from start to end
+    std::lock_guard<std::mutex> lock(g_pipe[dev].mu);
+    HIP_TRY(hipDeviceSynchronize());
     HIP_TRY(hipMemcpyToSymbol(HIP_SYMBOL(g_spin_limit), &v, sizeof(int)));
     return I6FBW_OK;
 }

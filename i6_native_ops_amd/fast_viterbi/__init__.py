@@ -8,6 +8,8 @@ from typing import Tuple
 
 import torch
 
+from .._version import __version__  # noqa: F401  (fast_viterbi/__init__.py:8 of the reference)
+
 try:
     from . import fast_viterbi_core as core
 except ImportError as exc:  # pragma: no cover - depends on the build state

@@ -14,6 +14,8 @@ from typing import Tuple
 
 import torch  # noqa: F401  (libtorch must be loaded before the extension)
 
+from .._version import __version__  # noqa: F401  (fbw/__init__.py:8 of the reference)
+
 try:
     from . import fbw_core as core
 except ImportError as exc:  # pragma: no cover

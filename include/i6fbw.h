@@ -34,7 +34,13 @@ enum {
                                              state ids spread over nearly 2*edges ids) */
     I6FBW_ERR_BAD_INDEX = -14,            /* device-side: sequence, emission or state index out of range */
     I6FBW_ERR_TIMEOUT = -15,              /* device-side: a stage gave up waiting for another stage of the call */
-    I6FBW_ERR_STATIC_WORKSPACE = -16      /* i6fbw_run_static: the problem needs more than I6FBW_STATIC_WORKSPACE_BYTES */
+    I6FBW_ERR_STATIC_WORKSPACE = -16,     /* i6fbw_run_static: the problem needs more than I6FBW_STATIC_WORKSPACE_BYTES */
+    /* Retired: earlier versions of this header refused what the general path now handles.  The names stay so that
+       code written against them still compiles; the library never returns these values any more. */
+    I6FBW_ERR_F_TOO_LARGE = -4,
+    I6FBW_ERR_SEQ_TOO_MANY_EDGES = -10,
+    I6FBW_ERR_SEQ_SPARSE_STATES = -11,
+    I6FBW_ERR_SEQ_DEGREE = -12
 };
 
 /* Layout of the posterior tensor written by i6fbw_run. */
@@ -130,7 +136,11 @@ int i6fbw_run_strided(const float* am_scores, int64_t am_stride_t, int64_t am_st
  * with I6FBW_ERR_STATIC_WORKSPACE.  All calls on one GPU share the one buffer: calls that overlap
  * in time on the same GPU (two streams, two host threads) race; calls on one stream are ordered
  * and safe.  i6fbw_static_workspace hands out the buffer of the current device, e.g. for
- * i6fbw_read_status(buffer, B, stream, ...) after a call.
+ * i6fbw_read_status(buffer, B, stream, ...) after a call.  The first use of either function on a device
+ * sets kernel attributes and takes the buffer's address there: under graph capture, call
+ * i6fbw_static_workspace (or make one eager call) before the capture begins.  The buffer is part of the
+ * library's code object: 32 MiB of every GPU the library is used on are taken from the moment it is
+ * loaded there, whether or not this entry point is ever called.
  */
 #define I6FBW_STATIC_WORKSPACE_BYTES (32u << 20)
 int i6fbw_run_static(const float* am_scores, int64_t am_stride_t, int64_t am_stride_b,
@@ -219,11 +229,14 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
 void i6fbw_set_overlap(int mode);
 
 /*
- * Kernels of the overlapped schedule that wait for another kernel of the same call poll at most
- * `polls` times (default 2^20, restored by polls <= 0) before they give up: the call then reports
- * I6FBW_ERR_TIMEOUT and the rows that could not be computed hold NaN.  Device-wide for the current
- * device; it exists so that a test can force that path from the host (polls = 1) while every kernel
- * still runs to its normal end.  No counterpart in the reference.
+ * TEST HOOK, not for production code.  Kernels of the overlapped schedule that wait for another kernel
+ * of the same call poll at most `polls` times (default 2^20, restored by polls <= 0) before they give up:
+ * the call then reports I6FBW_ERR_TIMEOUT and the rows that could not be computed hold NaN.  It exists so
+ * that a test can force that path from the host (polls = 1) while every kernel still runs to its normal
+ * end.  Device-wide for the current device: the call waits for the device to go idle, takes the lock that
+ * serialises the library's calls on it, and changes the limit for every call enqueued afterwards by any
+ * thread -- a thread that calls i6fbw_run on the same device at the same time gets either limit.
+ * No counterpart in the reference.
  */
 int i6fbw_set_spin_limit(int polls);
 

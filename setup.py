@@ -38,9 +38,15 @@ class BinaryDistribution(Distribution):
         return True
 
 
+def _version():
+    scope = {}
+    exec(open(os.path.join(TOP, "i6_native_ops_amd", "_version.py")).read(), scope)
+    return scope["__version__"]
+
+
 setup(
     name="i6_native_ops_amd",
-    version="0.2.0",
+    version=_version(),
     description="Full-sum forward-backward (FBW) loss and best-path alignment of rwth-i6/i6_native_ops for AMD MI355X (gfx950)",
     packages=find_packages(include=["i6_native_ops_amd", "i6_native_ops_amd.*"]),
     package_data={"i6_native_ops_amd": ["csrc/*.hip", "csrc/*.inc", "csrc/*.cpp", "csrc/*.h", "fbw/*.so", "fast_viterbi/*.so"]},

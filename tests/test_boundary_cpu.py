@@ -111,6 +111,35 @@ def test_packaging_metadata():
     assert "out_root" in inspect.signature(build.build_all).parameters
 
 
+@pytest.mark.slow
+def test_build_step_of_the_install_produces_a_loadable_package(tmp_path):
+    """What `pip install --no-build-isolation .` runs (the reference: setup.py:25-64 through torch's BuildExtension):
+    setup.py's build step into a scratch build tree, then the C-ABI library of that tree is loaded and exports every
+    symbol the header declares, and the tree holds both PyTorch bindings and the version.  Compiles everything:
+    minutes."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    build_lib = tmp_path / "lib"
+    subprocess.check_call([sys.executable, "setup.py", "-q", "build_py", "-b", str(build_lib)], cwd=root,
+                          stdout=subprocess.DEVNULL)
+    pkg = build_lib / "i6_native_ops_amd"
+    assert (pkg / "fbw" / "libi6fbw.so").exists()
+    assert list((pkg / "fbw").glob("fbw_core*.so")) and list((pkg / "fast_viterbi").glob("fast_viterbi_core*.so"))
+    # a fresh interpreter that sees the build tree only
+    code = ("import sys; sys.path.insert(0, %r); import i6_native_ops_amd; from i6_native_ops_amd import cabi; "
+            "assert cabi.__file__.startswith(%r), cabi.__file__; lib = cabi.load(); "
+            "missing = [s for s in cabi.SYMBOLS if not hasattr(lib, s)]; assert not missing, missing; "
+            "print(i6_native_ops_amd.__version__)") % (str(build_lib), str(build_lib))
+    out = subprocess.check_output([sys.executable, "-c", code], cwd=str(tmp_path), text=True)
+    from i6_native_ops_amd import __version__
+    assert out.strip() == __version__
+
+
+DENSE_SCRATCH_ALONE = 32      # bytes per lane of fbw_recurse_dense<false>
+
+
 def test_kernels_stay_within_their_register_budgets():
     """The build records what the compiler reports for every kernel.  The dense writer is launched for eight waves per
     SIMD (64 registers) and the gather, the preparation and the recursion instance for small batches are written to
@@ -123,6 +152,10 @@ def test_kernels_stay_within_their_register_budgets():
     if not os.path.exists(path):
         pytest.skip("kernel_resources.json is written by `python -m i6_native_ops_amd.build`")
     res = json.load(open(path))
+    # the record belongs to the sources that are here (it is rewritten by every build)
+    from i6_native_ops_amd import build
+    assert res.get("_sources_sha256") == build.sources_digest(), \
+        "kernel_resources.json was made from other kernel sources: rebuild (python -m i6_native_ops_amd.build)"
 
     def kernels(fragment):
         found = {k: v for k, v in res.items() if fragment in k}
@@ -137,7 +170,21 @@ def test_kernels_stay_within_their_register_budgets():
     for fragment in ("fbw_gather", "fbw_prepare", "fbw_padfill", "fbw_scan_sorted", "11fbw_recurseI", "vit_align"):
         for name, r in kernels(fragment).items():
             assert r["scratch"] == 0, (name, r)
-    for name, r in kernels("fbw_recurse_dense").items():
-        assert r["vgprs"] <= 104, (name, r)          # two workgroups per compute unit and room for the gather's waves
     for name, r in kernels("fbw_recurse_big").items():
-        assert r["vgprs"] <= 128, (name, r)          # sixteen waves per compute unit
+        assert r["vgprs"] <= 128 and r["scratch"] == 0, (name, r)          # sixteen waves per compute unit
+    for name, r in kernels("fbw_combine").items():
+        if name.endswith("Lb1EEEvNS_8CombArgsE"):
+            # the instance for the -log output: a few reloads per frame on its paths for sequences of more than 1024
+            # edges, none on the path for smaller ones (with two waves per SIMD it needs none and small sequences lose)
+            assert r["vgprs"] <= 168 and r["scratch"] <= 124, (name, r)
+        else:
+            assert r["vgprs"] <= 168 and r["scratch"] == 0, (name, r)      # three waves per SIMD beside a 48 KB row image
+    for name, r in kernels("fbw_recurse_dense").items():
+        if "ILb0E" in name:
+            # stage after stage: two workgroups have a compute unit's registers to themselves; what is left in scratch
+            # belongs to the rarely used loop bodies for several states per thread
+            assert r["vgprs"] <= 128 and r["scratch"] <= DENSE_SCRATCH_ALONE, (name, r)
+        else:
+            # beside gather and dense write (a schedule only a test switch selects for such batches): 96 registers, so
+            # that their waves find room; the loop bodies for several states per thread pay with spills
+            assert r["vgprs"] <= 104 and r["scratch"] <= 264, (name, r)

@@ -165,6 +165,58 @@ def test_one_large_automaton_of_higher_degree_among_small_ones(oracle):
     assert not failures, failures
 
 
+class _Args:
+    """the fields of a workload that check() reads"""
+    def __init__(self, am, edges, weights, se, lens, n_states):
+        self.am_scores, self.edges, self.weights, self.start_end_states, self.seq_lens, self.n_states = am, edges, weights, se, lens, n_states
+
+
+# bounds of the two groups below: just above what they measure today
+PERMUTED_IDS_BOUND = 1e-4
+TIGHT_MONOPHONE_BOUND = 1e-4
+
+
+@pytest.mark.parametrize("companions", [0, 90], ids=["large_automata_instance", "two_per_unit_instance"])
+@pytest.mark.parametrize("shuffle", [False, True], ids=["edges_in_order", "edges_shuffled"])
+def test_tight_chains_under_arbitrary_state_ids(oracle, companions, shuffle):
+    """Forty chains of 1021 states over 1021 to 1100 frames whose state ids are drawn at random from a range three times
+    as large: nothing about the ids says where a state sits in its automaton.  The renormalisation of the stored
+    rows has to find the states that can still matter from the automaton itself (this shape had the worst
+    posterior error of all random runs, 9.3e-5, while it looked at the ids).  Alone the batch runs the recursion
+    instance for large automata, with ninety small sequences beside it the one of which two workgroups share a
+    compute unit."""
+    from tests.helpers import spread_state_ids
+    from tests.test_flat_writer_gpu import merge
+    T = 1100
+    parts = [make_workload("cart", seed=955309586, T=T, B=40, F=97, n_labels=(340, 340), shuffle_edges=shuffle)]
+    parts[0].seq_lens[:] = np.resize(np.asarray([1100, 1021, 1098, 1050, 1030, 1075, 1023], dtype=np.int32), 40)
+    if companions:
+        parts.insert(0, make_workload("monophone", seed=371914332, T=T, B=companions, F=97, n_labels=(3, 3), shuffle_edges=True))
+        parts[0].seq_lens[:] = T
+    am, edges, weights, se, lens, n_states = merge(parts)
+    edges, se, n_states = spread_state_ids(edges, se, n_states, "permute", seed=17)
+    failures, worst = [], 0.0
+    for overlap in (0, 1):
+        worst = max(worst, check(oracle, _Args(am, edges, weights, se, lens, n_states), overlap,
+                                 f"40 chains of 1021 states, permuted ids, {companions} small beside them, shuffle={shuffle}, overlap={overlap}",
+                                 failures))
+    assert not failures, failures
+    assert worst <= PERMUTED_IDS_BOUND
+
+
+def test_large_batch_of_tight_monophone_automata(oracle):
+    """140 monophone automata of 200 to 400 states over 320 to 400 frames, many of them with barely more frames than
+    states, in one batch: the recursion instance of which two workgroups share a compute unit, whose sequences of
+    fewer than 384 frames used to keep float state vectors whatever their shape (8.7e-5 in the random runs)."""
+    W = make_workload("monophone", seed=14440930, T=400, B=140, F=97, n_labels=(67, 133), shuffle_edges=True)
+    # (lengths as drawn, 320 to 400 frames: about a third of the automata have a path at all, most of those a tight one)
+    failures, worst = [], 0.0
+    for overlap in (0, 1):
+        worst = max(worst, check(oracle, W, overlap, f"140 tight monophone automata, overlap={overlap}", failures))
+    assert not failures, failures
+    assert worst <= TIGHT_MONOPHONE_BOUND
+
+
 def test_random_shapes(oracle):
     """160 random cases: family, size, tightness of the alignment, edge order, batch size, schedule."""
     rng = np.random.default_rng(20241)

@@ -82,3 +82,46 @@ def test_too_large_is_refused():
         cabi.run_static(256, 32 * 12001, 12001, 256, 30000, 256, 256, 32, 256, 1000, 32, 12001, 30000, 12000, 0, 256, 256, 0)
     assert e.value.code == cabi.ERR_STATIC_WORKSPACE
     assert "32 MiB" in str(e.value)
+
+
+def test_captured_into_a_graph_and_replayed(oracle):
+    """The callers the entry point is for include code under HIP graph capture: the call is captured (after
+    i6fbw_static_workspace has set the device up -- kernel attributes and the address of the built-in buffer are taken at
+    the first use on a device, which must not fall into a capture), replayed three times with other work of the
+    library in between that dirties nothing it owns, and every replay gives what i6fbw_run gives eagerly."""
+    import torch
+    from i6_native_ops_amd import cabi
+    from tests.gpu_util import DeviceProblem
+    W = make_workload("monophone")
+    args = _slice(W, 200, 6)
+    p = DeviceProblem(*args)
+    want_out, want_loss = p.run(cabi.OUT_NEG_LOG)
+    want_out, want_loss = want_out.clone(), want_loss.clone()
+    cabi.static_workspace()                                 # device set-up outside the capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+
+    def call(stream):
+        cabi.run_static(p.am.data_ptr(), p.am.stride(0), p.am.stride(1), p.edges.data_ptr(), p.edges.stride(0),
+                        p.weights.data_ptr(), p.start_end.data_ptr(), p.start_end.stride(0), p.seq_lens.data_ptr(), p.T, p.B,
+                        p.F, p.E, p.n_states, cabi.OUT_NEG_LOG, p.out.data_ptr(), p.loss.data_ptr(), stream)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(side.cuda_stream)
+    other = DeviceProblem(*_slice(W, 120, 3))
+    for _ in range(3):
+        p.out.fill_(-7.0)
+        p.loss.fill_(-7.0)
+        # another problem through the built-in buffer between the replays: the captured call must not depend on
+        # what the buffer held when it was captured
+        call_stream = torch.cuda.current_stream().cuda_stream
+        cabi.run_static(other.am.data_ptr(), other.am.stride(0), other.am.stride(1), other.edges.data_ptr(), other.edges.stride(0),
+                        other.weights.data_ptr(), other.start_end.data_ptr(), other.start_end.stride(0), other.seq_lens.data_ptr(),
+                        other.T, other.B, other.F, other.E, other.n_states, cabi.OUT_PROB, other.out.data_ptr(),
+                        other.loss.data_ptr(), call_stream)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(p.loss, want_loss)
+        assert torch.equal(p.out, want_out)
