@@ -402,7 +402,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     unsigned* bitmap = lds + EB_MAX;
     int* wordpfx = (int*)(bitmap + ((a.F + 31) >> 5));
     __shared__ int wsum[NT / 64];
-    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin, s_count;
+    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin, s_count, s_nonmono, s_changed;
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -412,7 +412,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int32_t* e_seq = a.edges + 3 * a.edge_stride;
     const int E = a.E;
 
-    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; s_count = 0; }
+    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; s_count = 0; s_nonmono = 0; s_changed = 0; }
     __syncthreads();
     const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
     int unsorted = 0;
@@ -422,7 +422,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const bool sorted = s_sorted != 0;
 
     int edge_begin, n_edges, pos = 0;
-    int bad = 0;
+    int bad = 0, nonmono = 0;         // nonmono: some edge leads to a state with a smaller id
     unsigned mn = 0xffffffffu, mx = 0u;
     const int chunk = (E + NT - 1) / NT;
     const int lo = min(E, tid * chunk), hi = min(E, lo + chunk);
@@ -433,9 +433,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         for (int i = edge_begin + tid; i < edge_begin + n_edges; i += NT) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
             mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
+            nonmono |= t < f;
             if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
         }
         if (bad) atomicOr(&s_bad, 1);
+        if (nonmono) atomicOr(&s_nonmono, 1);
         if (mn <= mx) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
         __syncthreads();
     } else {
@@ -448,12 +450,14 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
                 eq++;
                 unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
                 mn = min(mn, min(f, t)); mx = max(mx, max(f, t));
+                nonmono |= t < f;
                 if (f >= (unsigned)a.n_states || t >= (unsigned)a.n_states || (unsigned)e_emis[i] >= (unsigned)a.F) bad = 1;
             }
             if (b == 0 && s >= (unsigned)a.B && s != 0xffffffffu) bad = 1;
         }
         if (lt) atomicAdd(&s_lt, lt);
         if (bad) atomicOr(&s_bad, 1);
+        if (nonmono) atomicOr(&s_nonmono, 1);
         if (eq) { atomicMin(&s_min, mn); atomicMax(&s_max, mx); }
         pos = block_excl_scan(eq, wsum, NT / 64, &n_edges);   // barriers inside publish the atomics too
         edge_begin = s_lt;
@@ -480,7 +484,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // sequence stays on the fast kernels: the 2n+2 ids fit the key array, and afterwards the n edge
     // keys its lower half and the distinct ids its upper half
     constexpr int RENUM_LDS_EDGES = EB_MAX / 2 - 1;
-    bool ranked = sparse && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
+    // The same renumbering serves sequences whose ids, spread or not, do not follow the automaton (some edge leads to a
+    // smaller id): their states are then numbered along the automaton (by_level below), which is what the recursion's
+    // renormalisation over live states and the activity band of the gather go by (live_window, min_steps).
+    const bool unordered = !err && n_edges > 0 && s_nonmono != 0 && s_bad == 0;
+    bool ranked = (sparse || unordered) && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
     if (sparse && !ranked) generic = 1;
     if (n_edges == 0) S = 1;
     if (!err && !sparse && S > S_MAX) generic = 1;
@@ -539,15 +547,66 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         }
         __syncthreads();
     }
-    // state id -> number within the sequence
-    auto local = [&](const unsigned id) -> unsigned {
-        if (!ranked) return id - smin;
+    // rank of a state id among the distinct ids of the sequence
+    auto rank_of = [&](const unsigned id) -> unsigned {
         int lo_ = 0, hi_ = (int)S;
         while (lo_ < hi_) {
             const int mid = (lo_ + hi_) >> 1;
             if (uniq[mid] < id) lo_ = mid + 1; else hi_ = mid;
         }
         return (unsigned)lo_;
+    };
+    // Numbers along the automaton for a sequence whose ids do not follow it: a state's level is the length of the
+    // longest path from the start state to it, self-loops aside (so every other edge leads to a higher level), and
+    // the states are numbered by level, then by id.  Levels come from repeated relaxation of all edges in LDS, one
+    // round per level at worst; an automaton with a cycle through several states has no such levels (the rounds do
+    // not come to rest within as many rounds as it has states) and keeps the ranks of its ids, as does one with more
+    // than LEVEL_STATES states.  Every role arrives at the same numbers.
+    constexpr int LEVEL_STATES = EB_MAX / 4;
+    int* level = (int*)(uniq + LEVEL_STATES);        // [S], later the number of the state with rank r
+    bool by_level = ranked && unordered && S <= LEVEL_STATES;
+    if (by_level) {
+        unsigned* pk = keys;                          // the edges as ranks: source | target << 16
+        for (int i = tid; i < n_edges; i += NT) {
+            const int e = edge_at(i);
+            pk[i] = rank_of((unsigned)e_from[e]) | (rank_of((unsigned)e_to[e]) << 16);
+        }
+        for (int r = tid; r < (int)S; r += NT) level[r] = -1;
+        __syncthreads();
+        if (tid == 0) level[rank_of(st_state)] = 0;
+        __syncthreads();
+        int round = 0;
+        for (; round <= (int)S; round++) {
+            bool changed = false;
+            for (int i = tid; i < n_edges; i += NT) {
+                const int u = (int)(pk[i] & 0xFFFFu), v = (int)(pk[i] >> 16);
+                const int lu = level[u];
+                if (u != v && lu >= 0 && level[v] < lu + 1) { atomicMax(&level[v], lu + 1); changed = true; }
+            }
+            // (the flag holds the last round that changed something, so it needs no reset and a round one barrier: a
+            // wave that is already in the next round can only raise it further)
+            if (changed) atomicMax(&s_changed, round + 1);
+            __syncthreads();
+            if (s_changed < round + 1) break;
+        }
+        __syncthreads();
+        if (round > (int)S) by_level = false;         // a cycle
+        else {
+            int N3 = NT;
+            while (N3 < (int)S) N3 <<= 1;
+            // states the start state does not reach come last
+            for (int i = tid; i < N3; i += NT) keys[i] = i < (int)S ? ((unsigned)(level[i] < 0 ? LEVEL_STATES : level[i]) << 12) | (unsigned)i : ~0u;
+            __syncthreads();
+            lds_bitonic_sort<NT>(keys, N3);
+            for (int i = tid; i < (int)S; i += NT) level[keys[i] & 0xFFFu] = i;
+            __syncthreads();
+        }
+    }
+    // state id -> number within the sequence
+    auto local = [&](const unsigned id) -> unsigned {
+        if (!ranked) return id - smin;
+        const unsigned r = rank_of(id);
+        return by_level ? (unsigned)level[r] : r;
     };
     int SP = (int)round16(S);
     if (!err && !generic && n_edges > 0) {
@@ -578,7 +637,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int DP = (int)round16(D > 0 ? D : 1);
 
     int start_loc = (int)local(st_state), end_loc = (int)local(en_state);
-    if (sparse && role == 2) {
+    if ((sparse || ranked) && role == 2) {
         // The general path looks the numbers up in an open-addressing table {id + 1, number} (see
         // local_state), which is written for every sequence with spread ids: the other two roles may
         // still send it there.  Numbers: the ranks from above, or, for a sequence too large for
@@ -644,7 +703,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         m->err = err ? err : (generic ? SEQ_GENERIC : 0);
         // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered;
         // bits 8 and up: see below
-        m->pad = (sorted ? 1 : 0) | (sparse ? 2 : 0);
+        m->pad = (sorted ? 1 : 0) | ((sparse || ranked) ? 2 : 0);
     }
     if (err || generic || n_edges == 0) {
         if (tid == 0) {
