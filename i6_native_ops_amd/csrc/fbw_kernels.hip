@@ -369,6 +369,7 @@ __device__ inline void lds_bitonic_sort(unsigned* keys, const int N) {
     }
 }
 
+constexpr int PREP_AUX_WORDS = 2048;   // scratch words of a preparation workgroup beside its sort keys
 constexpr int KEY_POS_BITS = 13;   // EB_MAX = 2^13 positions; the primary key sits above them
 static_assert((1 << KEY_POS_BITS) == EB_MAX, "key layout");
 
@@ -397,12 +398,13 @@ __device__ inline int min_steps(int from, int to, int dmax, int dmin) {
 // sequence starts; any other order is handled by a stable scan over the whole list.
 template <int NT>
 __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* lds) {
-    // dynamic LDS: sort keys, then the emission bitmap and its prefix counts (one word per 32 classes)
+    // dynamic LDS: sort keys, a scratch area (see by_level), then the emission bitmap and its prefix counts (one word per 32 classes)
     unsigned* keys = lds;
-    unsigned* bitmap = lds + EB_MAX;
+    unsigned* aux = lds + EB_MAX;
+    unsigned* bitmap = aux + PREP_AUX_WORDS;
     int* wordpfx = (int*)(bitmap + ((a.F + 31) >> 5));
     __shared__ int wsum[NT / 64];
-    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin, s_count, s_nonmono, s_changed;
+    __shared__ int s_lt, s_bad, s_kmax, s_sorted, s_dmax, s_dmin, s_count, s_nonmono;
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -412,7 +414,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int32_t* e_seq = a.edges + 3 * a.edge_stride;
     const int E = a.E;
 
-    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; s_count = 0; s_nonmono = 0; s_changed = 0; }
+    if (tid == 0) { s_lt = 0; s_bad = 0; s_kmax = 0; s_sorted = 1; s_min = 0xffffffffu; s_max = 0u; s_dmax = 0; s_dmin = 0; s_count = 0; s_nonmono = 0; }
     __syncthreads();
     const int nflag = (E + SCAN_BLOCK - 1) / SCAN_BLOCK;
     int unsorted = 0;
@@ -484,11 +486,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // sequence stays on the fast kernels: the 2n+2 ids fit the key array, and afterwards the n edge
     // keys its lower half and the distinct ids its upper half
     constexpr int RENUM_LDS_EDGES = EB_MAX / 2 - 1;
-    // The same renumbering serves sequences whose ids, spread or not, do not follow the automaton (some edge leads to a
-    // smaller id): their states are then numbered along the automaton (by_level below), which is what the recursion's
-    // renormalisation over live states and the activity band of the gather go by (live_window, min_steps).
-    const bool unordered = !err && n_edges > 0 && s_nonmono != 0 && s_bad == 0;
-    bool ranked = (sparse || unordered) && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
+    bool ranked = sparse && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
+    // Sequences whose ids, spread or not, do not follow the automaton (some edge leads to a smaller id) get numbers along
+    // the automaton where that matters (by_level below): that is what the recursion's renormalisation over live states
+    // and the activity band of the gather go by (live_window, min_steps).
+    const bool unordered = !err && n_edges > 0 && s_nonmono != 0 && s_bad == 0 && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
     if (sparse && !ranked) generic = 1;
     if (n_edges == 0) S = 1;
     if (!err && !sparse && S > S_MAX) generic = 1;
@@ -547,8 +549,9 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         }
         __syncthreads();
     }
-    // rank of a state id among the distinct ids of the sequence
+    // rank of a state id among the distinct ids of the sequence (ids that are not spread: place in their range)
     auto rank_of = [&](const unsigned id) -> unsigned {
+        if (!ranked) return id - smin;
         int lo_ = 0, hi_ = (int)S;
         while (lo_ < hi_) {
             const int mid = (lo_ + hi_) >> 1;
@@ -556,57 +559,80 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         }
         return (unsigned)lo_;
     };
-    // Numbers along the automaton for a sequence whose ids do not follow it: a state's level is the length of the
-    // longest path from the start state to it, self-loops aside (so every other edge leads to a higher level), and
-    // the states are numbered by level, then by id.  Levels come from repeated relaxation of all edges in LDS, one
-    // round per level at worst; an automaton with a cycle through several states has no such levels (the rounds do
-    // not come to rest within as many rounds as it has states) and keeps the ranks of its ids, as does one with more
-    // than LEVEL_STATES states.  Every role arrives at the same numbers.
-    constexpr int LEVEL_STATES = EB_MAX / 4;
-    int* level = (int*)(uniq + LEVEL_STATES);        // [S], later the number of the state with rank r
-    bool by_level = ranked && unordered && S <= LEVEL_STATES;
+    // Numbers along the automaton for a sequence whose ids do not follow it, where that matters: a tightly aligned one,
+    // fewer than five frames for every four states (chains of 1021 states over 1021-1100 frames came out at 9.9e-5 under
+    // permuted ids; the long-form configuration, whose optional states carry the highest ids, is at 2.5e-5 with 1.6
+    // frames per state and would pay 0.17 ms per call).  A state's height is the length of the longest path from it,
+    // self-loops aside, so every other edge leads to a lower state, and the states are numbered by falling height, then
+    // by id.  Heights by policy iteration: every state picks the highest of its successors, the heights along the chosen
+    // chains are added up by pointer jumping (log2 S rounds), and the states pick again, until every state sits exactly
+    // one above its highest successor -- two or three picks for a chain with optional states, whatever the order of
+    // ids and edges (one round per state, as relaxation needs, cost such a call a millisecond).  An automaton that has
+    // not come to rest after LEVEL_PICKS picks (a cycle through several states never does) keeps the ranks of its ids, as
+    // does one with more than LEVEL_STATES states.  Every role arrives at the same numbers.
+    constexpr int LEVEL_STATES = EB_MAX / 4, LEVEL_PICKS = 8;
+    static_assert(LEVEL_STATES <= PREP_AUX_WORDS && LEVEL_STATES <= 4096, "height << 16 | state; sort key height << 12 | state");
+    unsigned* dn = uniq + LEVEL_STATES;          // [S]: hops to the end of the chain of chosen successors << 16 | that end; later: the state's number
+    bool by_level = unordered && (ranked || !sparse) && !generic && S <= LEVEL_STATES && L > 0 && 5LL * S > 4LL * L;
     if (by_level) {
-        unsigned* pk = keys;                          // the edges as ranks: source | target << 16
+        unsigned* pk = keys;                      // the edges as ranks: source | target << 16
+        unsigned* cand = aux;                     // [S]: (height of the best successor + 1) << 16 | that successor
+        constexpr int SPT = LEVEL_STATES / NT;    // states per thread
+        const int nS = (int)S;
+        __syncthreads();        // the edge list written above (an edge list that is not grouped by sequence is read through it)
         for (int i = tid; i < n_edges; i += NT) {
             const int e = edge_at(i);
             pk[i] = rank_of((unsigned)e_from[e]) | (rank_of((unsigned)e_to[e]) << 16);
         }
-        for (int r = tid; r < (int)S; r += NT) level[r] = -1;
+        for (int r = tid; r < nS; r += NT) dn[r] = (unsigned)r;
         __syncthreads();
-        if (tid == 0) level[rank_of(st_state)] = 0;
-        __syncthreads();
-        int round = 0;
-        for (; round <= (int)S; round++) {
-            bool changed = false;
-            for (int i = tid; i < n_edges; i += NT) {
-                const int u = (int)(pk[i] & 0xFFFFu), v = (int)(pk[i] >> 16);
-                const int lu = level[u];
-                if (u != v && lu >= 0 && level[v] < lu + 1) { atomicMax(&level[v], lu + 1); changed = true; }
-            }
-            // (the flag holds the last round that changed something, so it needs no reset and a round one barrier: a
-            // wave that is already in the next round can only raise it further)
-            if (changed) atomicMax(&s_changed, round + 1);
+        bool rest = false;
+        for (int pick = 0; pick < LEVEL_PICKS && !rest; pick++) {
+            for (int r = tid; r < nS; r += NT) cand[r] = 0u;
             __syncthreads();
-            if (s_changed < round + 1) break;
+            for (int i = tid; i < n_edges; i += NT) {
+                const unsigned u = pk[i] & 0xFFFFu, w = pk[i] >> 16;
+                if (u != w) atomicMax(&cand[u], (((dn[w] >> 16) + 1u) << 16) | w);
+            }
+            __syncthreads();
+            int off = 0;
+            for (int r = tid; r < nS; r += NT) off |= (cand[r] >> 16) != (dn[r] >> 16);
+            if (!__syncthreads_or(off)) { rest = true; break; }
+            for (int r = tid; r < nS; r += NT) { const unsigned c = cand[r]; dn[r] = c ? (1u << 16) | (c & 0xFFFFu) : (unsigned)r; }
+            __syncthreads();
+            for (int span = 1; span < nS; span <<= 1) {
+                unsigned q[SPT];
+#pragma unroll
+                for (int j = 0; j < SPT; j++) {
+                    const int r = tid + j * NT;
+                    q[j] = 0u;
+                    if (r < nS) {
+                        const unsigned a_ = dn[r], b_ = dn[a_ & 0xFFFFu];
+                        q[j] = (min((a_ >> 16) + (b_ >> 16), 4095u) << 16) | (b_ & 0xFFFFu);      // (a cycle saturates and never comes to rest)
+                    }
+                }
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < SPT; j++)
+                    if (tid + j * NT < nS) dn[tid + j * NT] = q[j];
+                __syncthreads();
+            }
         }
-        __syncthreads();
-        if (round > (int)S) by_level = false;         // a cycle
+        if (!rest) by_level = false;
         else {
-            int N3 = NT;
-            while (N3 < (int)S) N3 <<= 1;
-            // states the start state does not reach come last
-            for (int i = tid; i < N3; i += NT) keys[i] = i < (int)S ? ((unsigned)(level[i] < 0 ? LEVEL_STATES : level[i]) << 12) | (unsigned)i : ~0u;
+            int N3 = 2;
+            while (N3 < nS) N3 <<= 1;
+            for (int i = tid; i < N3; i += NT) keys[i] = i < nS ? ((4095u - (dn[i] >> 16)) << 12) | (unsigned)i : ~0u;
             __syncthreads();
             lds_bitonic_sort<NT>(keys, N3);
-            for (int i = tid; i < (int)S; i += NT) level[keys[i] & 0xFFFu] = i;
+            for (int i = tid; i < nS; i += NT) dn[keys[i] & 0xFFFu] = (unsigned)i;
             __syncthreads();
         }
     }
     // state id -> number within the sequence
     auto local = [&](const unsigned id) -> unsigned {
-        if (!ranked) return id - smin;
         const unsigned r = rank_of(id);
-        return by_level ? (unsigned)level[r] : r;
+        return by_level ? dn[r] : r;
     };
     int SP = (int)round16(S);
     if (!err && !generic && n_edges > 0) {
@@ -637,12 +663,14 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int DP = (int)round16(D > 0 ? D : 1);
 
     int start_loc = (int)local(st_state), end_loc = (int)local(en_state);
-    if ((sparse || ranked) && role == 2) {
+    if ((sparse || by_level) && role == 2) {
         // The general path looks the numbers up in an open-addressing table {id + 1, number} (see
-        // local_state), which is written for every sequence with spread ids: the other two roles may
-        // still send it there.  Numbers: the ranks from above, or, for a sequence too large for
-        // that, the order in which the ids happen to be entered (any numbering will do: the general
-        // path never compares ids, and the distance bounds of min_steps hold for every numbering).
+        // local_state), which is written for every sequence whose numbers are not simply the place of the
+        // id in its range: the other two roles may still send it there.  Numbers: the ones from above,
+        // or, for a sequence with spread ids that is too large for that, the order in which the ids happen
+        // to be entered (any numbering will do: the general path never compares ids, and the distance
+        // bounds of min_steps hold for every numbering).
+        const bool numbered = ranked || !sparse;
         int2* tab = a.renum + 2 * soff;
         const unsigned cap = renum_capacity(n_edges);
         for (unsigned i = tid; i < cap; i += NT) { store_agent(&tab[i].x, 0); store_agent(&tab[i].y, 0); }
@@ -652,7 +680,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
             unsigned h = renum_home(id, cap);
             while (true) {
                 const int seen = atomicCAS(&tab[h].x, 0, id + 1);
-                if (seen == 0) { store_agent(&tab[h].y, ranked ? (int)local((unsigned)id) : atomicAdd(&s_count, 1)); return; }
+                if (seen == 0) { store_agent(&tab[h].y, numbered ? (int)local((unsigned)id) : atomicAdd(&s_count, 1)); return; }
                 if (seen == id + 1) return;
                 h = h + 1 == cap ? 0 : h + 1;
             }
@@ -674,7 +702,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         if (tid == 0) { enter((int)st_state); enter((int)en_state); }
         wait_stores();
         __syncthreads();
-        if (!ranked) {
+        if (!numbered) {
             S = s_count;
             SP = (int)round16(S);
             start_loc = number_of((int)st_state);
@@ -703,7 +731,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         m->err = err ? err : (generic ? SEQ_GENERIC : 0);
         // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered;
         // bits 8 and up: see below
-        m->pad = (sorted ? 1 : 0) | ((sparse || ranked) ? 2 : 0);
+        m->pad = (sorted ? 1 : 0) | ((sparse || by_level) ? 2 : 0);
     }
     if (err || generic || n_edges == 0) {
         if (tid == 0) {
@@ -2916,7 +2944,7 @@ std::mutex g_mutex;           // process-wide settings and the stage profile
 static __device__ __align__(256) unsigned char g_static_workspace[I6FBW_STATIC_WORKSPACE_BYTES];
 
 // LDS of a preparation workgroup: sort keys, emission bitmap and its prefix counts
-size_t prep_lds_bytes(int F) { return (size_t)EB_MAX * 4 + (F <= F_BITMAP_MAX ? (size_t)((F + 31) >> 5) * 8 : 0); }
+size_t prep_lds_bytes(int F) { return (size_t)(EB_MAX + PREP_AUX_WORDS) * 4 + (F <= F_BITMAP_MAX ? (size_t)((F + 31) >> 5) * 8 : 0); }
 
 // 1024-thread workgroups sort fastest, but only two of them fit on a compute unit: batches that
 // would need a second round of them take 512-thread workgroups, four to a unit.

@@ -122,7 +122,7 @@ def test_build_step_of_the_install_produces_a_loadable_package(tmp_path):
     import sys
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     build_lib = tmp_path / "lib"
-    subprocess.check_call([sys.executable, "setup.py", "-q", "build_py", "-b", str(build_lib)], cwd=root,
+    subprocess.check_call([sys.executable, "setup.py", "-q", "build_py", "--build-lib", str(build_lib)], cwd=root,
                           stdout=subprocess.DEVNULL)
     pkg = build_lib / "i6_native_ops_amd"
     assert (pkg / "fbw" / "libi6fbw.so").exists()
