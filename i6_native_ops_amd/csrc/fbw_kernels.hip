@@ -408,6 +408,11 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     __shared__ unsigned s_min, s_max;
 
     const int role = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    // what depends on nothing but the sequence index is requested before anything is waited for (seq_first / seq_next: where
+    // the edges of this sequence and of the next one begin if the list is grouped by sequence, see fbw_scan_sorted)
+    const int seq_first = a.E > 0 ? a.seqbegin[b] : 0, seq_next = a.E > 0 ? a.seqbegin[b + 1] : 0;
+    const unsigned st_state = (unsigned)a.start_end[b], en_state = (unsigned)a.start_end[a.se_stride + b];
+    const unsigned sl = (unsigned)a.seq_lens[b];
     const int32_t* e_from = a.edges;
     const int32_t* e_to = a.edges + a.edge_stride;
     const int32_t* e_emis = a.edges + 2 * a.edge_stride;
@@ -429,8 +434,8 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int chunk = (E + NT - 1) / NT;
     const int lo = min(E, tid * chunk), hi = min(E, lo + chunk);
     if (sorted) {
-        edge_begin = E > 0 ? a.seqbegin[b] : 0;
-        n_edges = E > 0 ? a.seqbegin[b + 1] - edge_begin : 0;
+        edge_begin = seq_first;
+        n_edges = seq_next - seq_first;
         if (b == 0 && E > 0 && (unsigned)e_seq[E - 1] >= (unsigned)a.B && (unsigned)e_seq[E - 1] != 0xffffffffu) bad = 1;
         for (int i = edge_begin + tid; i < edge_begin + n_edges; i += NT) {
             unsigned f = (unsigned)e_from[i], t = (unsigned)e_to[i];
@@ -465,7 +470,6 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         edge_begin = s_lt;
     }
 
-    const unsigned st_state = (unsigned)a.start_end[b], en_state = (unsigned)a.start_end[a.se_stride + b];
     unsigned smin = min(min(s_min, st_state), en_state), smax = max(max(s_max, st_state), en_state);
     int err = 0;
     if (s_bad || st_state >= (unsigned)a.n_states || en_state >= (unsigned)a.n_states) err = I6FBW_ERR_BAD_INDEX;
@@ -473,7 +477,6 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // generic_viterbi).
     int generic = 0;
     if (!err && n_edges > EB_MAX) generic = 1;
-    const unsigned sl = (unsigned)a.seq_lens[b];
     // full sum: a length outside [1, T] leaves the sequence without probability mass; best path:
     // lengths beyond T are read as T
     const int L = a.best_path ? ((int)sl < 0 ? 0 : min((int)sl, a.T)) : ((sl >= 1u && sl <= (unsigned)a.T) ? (int)sl : 0);
@@ -884,8 +887,13 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         constexpr int EPT = EB_MAX / NT;
         int slot_[EPT], from_[EPT], upto_[EPT];     // slot of my edges (-1: none), first and last live frame
 #pragma unroll
+        for (int j = 0; j < EPT; j++) { slot_[j] = -1; from_[j] = 0; upto_[j] = -1; }
+#pragma unroll
         for (int j = 0; j < EPT; j++) {
-            slot_[j] = -1; from_[j] = 0; upto_[j] = -1;
+            // (the whole workgroup leaves at the first round without edges: a sequence of a few hundred edges has one or
+            // two, and every further one cost a microsecond although no lane had anything to do in it -- 15 of the 37 us
+            // of the preparation of 256 CTC automata)
+            if (j * NT >= n_edges) break;
             if (tid + j * NT < n_edges) {
                 const unsigned key = keys[tid + j * NT];
                 const int e = edge_at((int)(key & POS_MASK));
@@ -920,6 +928,7 @@ template <int NT>
 __global__ __launch_bounds__(NT) void fbw_prepare(PrepArgs a) {
     extern __shared__ unsigned prep_lds[];
     prepare_sequence<NT>(a, prep_lds);      // every exit from it is taken by the whole workgroup
+
     // The recursion kernel of the overlapped schedule is already on the machine and waits for this
     // count: write this workgroup's tables back from the L2 of its XCD before it is raised.
     __syncthreads();
