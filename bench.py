@@ -85,6 +85,25 @@ def cpu_threads(W, fbw_oracle):
     return max(1, min(W.B, cores, fbw_oracle.max_threads()))
 
 
+def committed_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary of this workload (counters need the
+    profiler, so they are not measured in this run), the name of that summary, and whether it was made from other kernel
+    sources than the ones here (it records their digest)."""
+    tpath = os.path.join(ROOT, "profiles", f"fbw_{workload}_hbm_traffic.txt")
+    if not os.path.exists(tpath):
+        return None, None, None
+    import re
+    text = open(tpath).read()
+    m = re.search(kernel + r", scaled:.*= ([0-9.]+) MB per launch", text)
+    if not m:
+        return None, None, None
+    from i6_native_ops_amd import build
+    d = re.search(r"kernel sources sha256: ([0-9a-f]+)", text)
+    stale = not (d and d.group(1) == build.sources_digest())
+    return (int(float(m.group(1)) * 1e6),
+            f"profiles/fbw_{workload}_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, committed)", stale)
+
+
 def per_config_entry(name, headline=None):
     """Timing and parity of one benchmark configuration (the headline's device problem is reused)."""
     import numpy as np
@@ -112,7 +131,11 @@ def per_config_entry(name, headline=None):
     out = P.out.cpu().numpy()
     for t0 in range(0, W.T, 64):          # in slices: exp of the whole oracle tensor at once doubles the host memory
         post_err = max(post_err, float(np.max(np.abs(out[t0:t0 + 64] - np.exp(-want_out[t0:t0 + 64].astype(np.float64))))))
+    from i6_native_ops_amd import cabi
+    writer = "fbw_flat" if cabi.last_dense_writer() == 1 else "fbw_combine"
+    traffic, _, stale = committed_traffic(name, writer)
     return {"T": W.T, "B": W.B, "F": W.F, "E": W.E, "ms_median": round(med, 4), "ms_min": round(mn, 4),
+            "dense_writer": writer, "dense_writer_traffic": traffic, "traffic_stale": stale,
             "neg_log_ms_median": round(neg_log[len(neg_log) // 2], 4),
             "algorithmic_bytes": alg, "gbps": round(alg / (med * 1e-3) / 1e9, 1),
             "frac_of_hbm_peak": round(alg / (med * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -132,6 +155,8 @@ def main():
     ap.add_argument("--no-per-config", action="store_true",
                     help="skip the per-configuration table (timings and errors against the oracle for all five workloads)")
     ap.add_argument("--out-mode", type=int, default=1, help="0: -log posterior with +inf holes, 1: posterior")
+    ap.add_argument("--no-other-mode", action="store_true",
+                    help="skip the timing of the other output mode (a profile of the run then holds the kernels of one mode only)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise copy kernel over 1 GiB (3 times) so that a rocprofv3 --pmc run of "
                          "this command shows what FETCH_SIZE / WRITE_SIZE read for a known amount of traffic")
@@ -201,14 +226,7 @@ def main():
     comb_gbps = comb_bytes / (comb_ms * 1e-3) / 1e9 if comb_ms > 0 else 0.0
     # HBM bytes per launch of that kernel: not measured in this run (counters need the profiler); the
     # figure comes from the committed rocprofv3 --pmc summary of this command and names it
-    traffic, traffic_source = None, None
-    tpath = os.path.join(ROOT, "profiles", f"fbw_{args.workload}_hbm_traffic.txt")
-    if os.path.exists(tpath):
-        import re
-        m = re.search(kernel + r", scaled:.*= ([0-9.]+) MB per launch", open(tpath).read())
-        if m:
-            traffic = int(float(m.group(1)) * 1e6)
-            traffic_source = f"profiles/fbw_{args.workload}_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, committed)"
+    traffic, traffic_source, traffic_stale = committed_traffic(args.workload, kernel)
 
     result = {
         "metric": f"FBW loss+grad ms/call + achieved HBM GB/s at T={W.T},B={W.B},F={W.F} fp32",
@@ -232,20 +250,21 @@ def main():
                    "stage_ms": {k: round(v, 4) for k, v in zip(cabi.STAGE_NAMES, stage_ms)}},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(comb_gbps, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(comb_gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "traffic_source": traffic_source,
+                     "traffic_source": traffic_source, "traffic_stale": traffic_stale,
                      "algorithmic_bytes_per_launch": comb_bytes, "kernel_ms_per_launch": round(comb_ms, 4)},
     }
 
     # the other output mode of the same call (informational): -log posteriors with +inf holes, as the reference's binding
     # fbw_core.fbw returns them (fbw_op.cu:366-377,392), when the timed mode is the posterior, and the other way round
-    other = Problem.__new__(Problem)
-    other.__dict__.update(P.__dict__)
-    other.out_mode = 0 if args.out_mode == 1 else 1
-    ot = other.single_call_times(20, 5)
-    result["config"]["neg_log_ms" if args.out_mode == 1 else "posterior_ms"] = round(ot[len(ot) // 2], 4)
-    if args.out_mode == 1:
-        step()      # the headline problem's buffers hold the posterior mode's results again (the per-config table checks them)
-        torch.cuda.synchronize()
+    if not args.no_other_mode:
+        other = Problem.__new__(Problem)
+        other.__dict__.update(P.__dict__)
+        other.out_mode = 0 if args.out_mode == 1 else 1
+        ot = other.single_call_times(20, 5)
+        result["config"]["neg_log_ms" if args.out_mode == 1 else "posterior_ms"] = round(ot[len(ot) // 2], 4)
+        if args.out_mode == 1:
+            step()      # the headline problem's buffers hold the posterior mode's results again (the per-config table checks them)
+            torch.cuda.synchronize()
 
     # wrapper level (informational): fbw_loss(log_probs[B,T,F]).sum().backward() with the fused front end
     # and with the reference's literal neg/transpose/contiguous/exp chain around the same kernels

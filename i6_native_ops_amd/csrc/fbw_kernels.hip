@@ -1765,6 +1765,7 @@ struct CombArgs {
     int* sync;
     int tile_w;                  // 0: the row image holds the whole row; else its width in floats (a multiple of 32), see finish_row
     int direct_only;             // beside fbw_flat: only the sequences that kernel leaves to this one (flat_direct)
+    int small_elsewhere = 0;     // the sequences of comb_small() are written by the SMALL instance of this kernel, launched beside this one
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1945,8 +1946,23 @@ __device__ __forceinline__ float neg_log_value(const LogSum s, const float mn, c
 // (At three waves per SIMD the -log instance keeps a few values of its paths for sequences of more than 1024 edges
 // in scratch memory -- six reloads per frame there, none on the path for smaller sequences; at two it needs none, and
 // the monophone configuration, all of whose sequences are small, takes 8 % longer per call.)
-template <bool SYNC, bool NEGLOG>
-__global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
+// SMALL: the instance for the sequences whose edges and slots stay in a thread's registers over a strip (comb_small: up
+// to 1024 edges and 512 distinct emissions) and nothing else.  It needs a third of the registers, so that COMB_SMALL_OCC
+// workgroups share a compute unit instead of three: a strip is a chain of dependent round trips (operands of a frame,
+// block minimum, staging area, per-emission sums, block sum, row image, row out), and what hides them is the number of
+// strips in flight -- with short rows (the row writer's domain: F below 2048 or a small tensor) the strips of a whole
+// batch then run at the same time (monophone configuration: dense write 58 -> 42 us, call 0.194 -> 0.178 ms; four or six
+// workgroups per unit measure the same, eight need 64 registers and spill: 50 us).  The host launches it next to the
+// general instance, which leaves those sequences out (small_elsewhere).
+__device__ __forceinline__ bool comb_small(const SeqMeta& m) {
+    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= COMB_XS && m.D <= 2 * COMB_THREADS;
+}
+#ifndef I6_COMB_SMALL_OCC
+#define I6_COMB_SMALL_OCC 6
+#endif
+constexpr int COMB_SMALL_OCC = I6_COMB_SMALL_OCC;
+template <bool SYNC, bool NEGLOG, bool SMALL = false>
+__global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_combine(CombArgs a) {
     extern __shared__ float4a lds4[];
     __shared__ float redmin[COMB_THREADS / 64];
     __shared__ float redsum[COMB_THREADS / 64];
@@ -1960,6 +1976,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
     const SeqMeta m = a.meta[b];
     if (m.L == 0) return;                                      // fbw_padfill has written every row
     if (a.direct_only && !flat_direct(m)) return;
+    if (SMALL ? !comb_small(m) : (a.small_elsewhere && comb_small(m))) return;
     const int T = a.T, B = a.B, F = a.F;
     // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
     // forward and the backward recursion meet, so those rows are complete first
@@ -1971,7 +1988,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
 #ifdef I6_TRACE
     if (tid == 0) { atomicMin(&g_trace[2], wall_clock64()); if (b == 0) g_trace[1024 + strip] = wall_clock64(); }
 #endif
-    if (seq_error(m) < 0 || m.n_edges == 0) {
+    if (!SMALL && (seq_error(m) < 0 || m.n_edges == 0)) {
         // no recursion ran for this sequence: NaN for a reported problem, empty frames otherwise
         const bool err = seq_error(m) != 0;
         const float v = err ? __builtin_nanf("") : (a.out_mode != I6FBW_OUT_NEG_LOG ? 0.f : INF_F);
@@ -2007,7 +2024,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             return;
         }
     }
-    if (seq_error(m) > 0) {
+    if (!SMALL && seq_error(m) > 0) {
         __shared__ float gred[32];
         const long long soff = state_off(m.edge_begin, b);
         generic_combine<SYNC>(a.gen, m, b, t0, tv, T, B, F, a.out_mode, a.alpha + (size_t)T * soff, a.beta + (size_t)T * soff,
@@ -2047,7 +2064,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
         const float inv = dead ? 0.f : psign / tot;
         float* orow = a.out + t * a.ost_t + b * a.ost_b;
         const int sh = row_misalign(orow);
-        if (a.tile_w) {
+        if (!SMALL && a.tile_w) {
             // Row longer than the image: tile after tile of the line-aligned view of the row (positions
             // sh .. sh+F-1 of base = orow - sh).  The slots are ordered by emission index, but every
             // thread simply looks which of its slots fall into the tile; after the tile has gone out
@@ -2099,7 +2116,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
         stream_image_row(orow, F, lds4, image);
     };
 
-    if (nE <= COMB_XS && D <= 2 * COMB_THREADS) {
+    if (SMALL || (nE <= COMB_XS && D <= 2 * COMB_THREADS)) {
         // fast path: this thread's edges and slots stay in registers for the whole strip, and
         // the operands of the next frame are fetched while the current one is processed
         constexpr int JE = COMB_XS / COMB_THREADS, JS = 2;
@@ -2166,7 +2183,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             if (!NEGLOG) tot = block_sum256(part, redsum);
             finish_row(t, mn, tot, sd, ls, em, JS, offs);
         }
-    } else if (nE <= COMB_MID_EDGES && D <= COMB_MID_SLOTS) {
+    } else if (!SMALL && nE <= COMB_MID_EDGES && D <= COMB_MID_SLOTS) {
         // medium sequences: this thread's edges still stay in registers for the whole strip (sixteen
         // of them, source and target packed), the operands of a frame are fetched in one go, and the
         // scores go through the LDS staging area in up to four passes
@@ -2234,7 +2251,7 @@ __global__ __launch_bounds__(COMB_THREADS, 3) void fbw_combine(CombArgs a) {
             const float tot = block_sum256(part, redsum);
             finish_row(t, mn, tot, sd, ls, em, JS, offs);
         }
-    } else {
+    } else if (!SMALL) {
         // general path: edge records re-read per frame, edges staged through LDS in passes of
         // COMB_XS, per-slot sums accumulated across the passes
         for (int t = t0; t < tv; t++) {
@@ -2964,10 +2981,17 @@ void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
 }
 
 // The dense writers, in the instance for the output mode (NEGLOG: the -log output, summed in log space)
+// (the row writer proper: first the instance for small sequences -- most batches are nothing else -- then the general
+// one for the rest; rows too long for the LDS image, and the sequences fbw_flat leaves over, are the general one's alone)
 template <bool SYNC>
-void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStream_t s, const CombArgs& ca) {
-    if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true>), grid, dim3(COMB_THREADS), lds, s, ca);
-    else hipLaunchKernelGGL((fbw_combine<SYNC, false>), grid, dim3(COMB_THREADS), lds, s, ca);
+void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStream_t s, CombArgs ca) {
+    if (!ca.direct_only && !ca.tile_w) {
+        if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, true>), grid, dim3(COMB_THREADS), lds, s, ca);
+        else hipLaunchKernelGGL((fbw_combine<SYNC, false, true>), grid, dim3(COMB_THREADS), lds, s, ca);
+        ca.small_elsewhere = 1;
+    }
+    if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, false>), grid, dim3(COMB_THREADS), lds, s, ca);
+    else hipLaunchKernelGGL((fbw_combine<SYNC, false, false>), grid, dim3(COMB_THREADS), lds, s, ca);
 }
 template <bool SYNC>
 void launch_flat(const bool neglog, const dim3 grid, hipStream_t s, const FlatArgs& fa) {
@@ -2985,8 +3009,10 @@ int device_init(Pipeline& p) {
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_recurse_dense<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(float) * REC_LDS_FLOATS_F32));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<1024>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
     HIP_TRY(hipFuncSetAttribute((const void*)fbw_prepare<512>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)prep_lds_bytes(F_BITMAP_MAX)));
-    for (const void* k : {(const void*)fbw_combine<true, false>, (const void*)fbw_combine<false, false>,
-                          (const void*)fbw_combine<true, true>, (const void*)fbw_combine<false, true>})
+    for (const void* k : {(const void*)fbw_combine<true, false, false>, (const void*)fbw_combine<false, false, false>,
+                          (const void*)fbw_combine<true, true, false>, (const void*)fbw_combine<false, true, false>,
+                          (const void*)fbw_combine<true, false, true>, (const void*)fbw_combine<false, false, true>,
+                          (const void*)fbw_combine<true, true, true>, (const void*)fbw_combine<false, true, true>})
         HIP_TRY(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
     hipFuncAttributes attr;
     HIP_TRY(hipFuncGetAttributes(&attr, (const void*)fbw_recurse_dense<true>));

@@ -173,9 +173,13 @@ def test_kernels_stay_within_their_register_budgets():
     for name, r in kernels("fbw_recurse_big").items():
         assert r["vgprs"] <= 128 and r["scratch"] == 0, (name, r)          # sixteen waves per compute unit
     for name, r in kernels("fbw_combine").items():
-        if name.endswith("Lb1EEEvNS_8CombArgsE"):
+        sync, neglog, small = (int(x) for x in re.search(r"fbw_combineILb(\d)ELb(\d)ELb(\d)E", name).groups())
+        if small:
+            # the instance for sequences of up to 1024 edges: six workgroups per compute unit
+            assert r["vgprs"] <= 80 and r["occupancy"] >= 6 and r["scratch"] <= (8 if neglog else 0), (name, r)
+        elif neglog:
             # the instance for the -log output: a few reloads per frame on its paths for sequences of more than 1024
-            # edges, none on the path for smaller ones (with two waves per SIMD it needs none and small sequences lose)
+            # edges (with two waves per SIMD it needs none and is slower)
             assert r["vgprs"] <= 168 and r["scratch"] <= 124, (name, r)
         else:
             assert r["vgprs"] <= 168 and r["scratch"] == 0, (name, r)      # three waves per SIMD beside a 48 KB row image
