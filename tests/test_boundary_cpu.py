@@ -24,6 +24,9 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(cabi.SYMBOLS)
     for n in names:
         assert getattr(lib, n) is not None
+    # the in-kernel timestamp hooks (-DI6_TRACE, a measurement build) are not part of the shipped library
+    for n in ("i6fbw_debug_trace", "i6fbw_debug_trace_set"):
+        assert not hasattr(lib, n), n
 
 
 def test_workspace_size_and_argument_validation():
