@@ -24,7 +24,7 @@ SYMBOLS = ("i6fbw_workspace_size", "i6fbw_run", "i6fbw_run_strided", "i6fbw_read
            "i6fbw_ctc_fsa_bounds", "i6fbw_build_ctc_fsa", "i6fbw_build_hmm_fsa",
            "i6fbw_profile_enable", "i6fbw_profile_read",
            "i6fbw_post_status", "i6fbw_poll_status", "i6fbw_set_status_mode", "i6fbw_get_status_mode",
-           "i6fbw_run_static", "i6fbw_static_workspace", "i6fbw_set_dense_writer", "i6fbw_last_dense_writer", "i6fbw_set_spin_limit")
+           "i6fbw_run_static", "i6fbw_static_workspace", "i6fbw_set_dense_writer", "i6fbw_last_dense_writer", "i6fbw_set_spin_limit", "i6fbw_set_band")
 STATIC_WORKSPACE_BYTES = 32 << 20
 ERR_STATIC_WORKSPACE = -16
 
@@ -91,6 +91,8 @@ def load():
         lib.i6fbw_set_overlap.restype = None
         lib.i6fbw_set_dense_writer.argtypes = [c.c_int]
         lib.i6fbw_set_dense_writer.restype = None
+        lib.i6fbw_set_band.argtypes = [c.c_int]
+        lib.i6fbw_set_band.restype = None
         lib.i6fbw_set_spin_limit.argtypes = [c.c_int]
         lib.i6fbw_set_spin_limit.restype = c.c_int
         lib.i6fbw_last_dense_writer.argtypes = []

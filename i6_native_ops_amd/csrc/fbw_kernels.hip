@@ -369,6 +369,60 @@ __device__ inline void lds_bitonic_sort(unsigned* keys, const int N) {
     }
 }
 
+// The same sort for N = R * NT keys with the keys in registers: thread tid holds the elements tid + r * NT.  Partners
+// NT or more apart sit in the same thread, partners less than a wave apart are reached with a lane exchange; only the
+// steps in between go through LDS (two barriers each): 18 of the 78 steps for 4096 keys on 1024 threads, where the
+// loop above has a barrier behind every step.  The caller has written the keys and passed a barrier; the sorted keys
+// are back in LDS behind the last barrier of this function.
+template <int NT, int R>
+__device__ __forceinline__ void bitonic_sort_in_registers(unsigned* keys, const int tid) {
+    unsigned x[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) x[r] = keys[tid + r * NT];
+    // a step with partners j < NT apart, for the stage of run length k
+    auto across_threads = [&](const int k, const int j) {
+        unsigned y[R];
+        if (j >= 64) {
+            __syncthreads();        // the reads of the step before (the initial ones on the first)
+#pragma unroll
+            for (int r = 0; r < R; r++) keys[tid + r * NT] = x[r];
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < R; r++) y[r] = keys[(tid ^ j) + r * NT];
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; r++) y[r] = (unsigned)__shfl_xor((int)x[r], j);
+        }
+        const bool lower = (tid & j) == 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const bool up = ((tid + r * NT) & k) == 0;
+            x[r] = (lower == up) ? min(x[r], y[r]) : max(x[r], y[r]);
+        }
+    };
+    for (int k = 2; k <= NT; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) across_threads(k, j);
+#pragma unroll
+    for (int kr = 2; kr <= R; kr <<= 1) {          // stages of run length kr * NT
+#pragma unroll
+        for (int jr = kr >> 1; jr > 0; jr >>= 1) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if ((r & jr) == 0) {
+                    const bool up = (r & kr) == 0;
+                    const unsigned lo = min(x[r], x[r | jr]), hi = max(x[r], x[r | jr]);
+                    x[r] = up ? lo : hi;
+                    x[r | jr] = up ? hi : lo;
+                }
+        }
+        for (int j = NT >> 1; j > 0; j >>= 1) across_threads(kr * NT, j);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; r++) keys[tid + r * NT] = x[r];
+    __syncthreads();
+}
+
 constexpr int PREP_AUX_WORDS = 2048;   // scratch words of a preparation workgroup beside its sort keys
 constexpr int KEY_POS_BITS = 13;   // EB_MAX = 2^13 positions; the primary key sits above them
 static_assert((1 << KEY_POS_BITS) == EB_MAX, "key layout");
@@ -489,19 +543,20 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // sequence stays on the fast kernels: the 2n+2 ids fit the key array, and afterwards the n edge
     // keys its lower half and the distinct ids its upper half
     constexpr int RENUM_LDS_EDGES = EB_MAX / 2 - 1;
-    bool ranked = sparse && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
     // Sequences whose ids, spread or not, do not follow the automaton (some edge leads to a smaller id) get numbers along
     // the automaton where that matters (by_level below): that is what the recursion's renormalisation over live states
     // and the activity band of the gather go by (live_window, min_steps).
     const bool unordered = !err && n_edges > 0 && s_nonmono != 0 && s_bad == 0 && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
+    // ... and such a sequence is ranked too when its ids, without being spread by the measure above, span more than the
+    // numbering below can hold, as the ids of one sequence among many do after a permutation over the whole batch (a chain
+    // of 1020 states with ids out of 3573, 1100 frames: 7.9e-5 before): the span says nothing about the number of states then
+    constexpr int LEVEL_STATES = EB_MAX / 4;
+    const bool span_too_wide = unordered && !sparse && S > LEVEL_STATES && L > 0 && 5LL * S > 4LL * L;
+    bool ranked = (sparse || span_too_wide) && n_edges <= RENUM_LDS_EDGES && !a.force_generic;
     if (sparse && !ranked) generic = 1;
     if (n_edges == 0) S = 1;
-    if (!err && !sparse && S > S_MAX) generic = 1;
+    if (!err && !sparse && !ranked && S > S_MAX) generic = 1;
     if (!err && a.force_generic && n_edges > 0) generic = 1;
-    // The recursion instance for batches of more sequences than half the compute units has room for
-    // double-precision state vectors of DENSE_F64_STATES states only: a larger sequence that needs them
-    // (recurse_workgroup) takes the general path, which keeps its vectors in double in memory.
-    if (!err && a.dense && !a.best_path && S > DENSE_F64_STATES && (5LL * S > 3LL * L || L > I6_FLOAT_FRAMES)) generic = 1;
     const long long soff = state_off(edge_begin, b), goff = slot_off(edge_begin, b);
 
     // i-th edge of this sequence in input order
@@ -552,6 +607,10 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         }
         __syncthreads();
     }
+    // The recursion instance for batches of more sequences than half the compute units has room for
+    // double-precision state vectors of DENSE_F64_STATES states only: a larger sequence that needs them
+    // (recurse_workgroup) takes the general path, which keeps its vectors in double in memory.
+    if (!err && a.dense && !a.best_path && S > DENSE_F64_STATES && (5LL * S > 3LL * L || L > I6_FLOAT_FRAMES)) generic = 1;
     // rank of a state id among the distinct ids of the sequence (ids that are not spread: place in their range)
     auto rank_of = [&](const unsigned id) -> unsigned {
         if (!ranked) return id - smin;
@@ -573,7 +632,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     // ids and edges (one round per state, as relaxation needs, cost such a call a millisecond).  An automaton that has
     // not come to rest after LEVEL_PICKS picks (a cycle through several states never does) keeps the ranks of its ids, as
     // does one with more than LEVEL_STATES states.  Every role arrives at the same numbers.
-    constexpr int LEVEL_STATES = EB_MAX / 4, LEVEL_PICKS = 8;
+    constexpr int LEVEL_PICKS = 8;
     static_assert(LEVEL_STATES <= PREP_AUX_WORDS && LEVEL_STATES <= 4096, "height << 16 | state; sort key height << 12 | state");
     unsigned* dn = uniq + LEVEL_STATES;          // [S]: hops to the end of the chain of chosen successors << 16 | that end; later: the state's number
     bool by_level = unordered && (ranked || !sparse) && !generic && S <= LEVEL_STATES && L > 0 && 5LL * S > 4LL * L;
@@ -666,7 +725,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
     const int DP = (int)round16(D > 0 ? D : 1);
 
     int start_loc = (int)local(st_state), end_loc = (int)local(en_state);
-    if ((sparse || by_level) && role == 2) {
+    if ((sparse || ranked || by_level) && role == 2) {
         // The general path looks the numbers up in an open-addressing table {id + 1, number} (see
         // local_state), which is written for every sequence whose numbers are not simply the place of the
         // id in its range: the other two roles may still send it there.  Numbers: the ones from above,
@@ -734,7 +793,7 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         m->err = err ? err : (generic ? SEQ_GENERIC : 0);
         // bit 0: the edges of the sequence are contiguous in the input; bit 1: its states are renumbered;
         // bits 8 and up: see below
-        m->pad = (sorted ? 1 : 0) | ((sparse || by_level) ? 2 : 0);
+        m->pad = (sorted ? 1 : 0) | ((sparse || ranked || by_level) ? 2 : 0);
     }
     if (err || generic || n_edges == 0) {
         if (tid == 0) {
@@ -788,20 +847,12 @@ __device__ __forceinline__ void prepare_sequence(const PrepArgs& a, unsigned* ld
         }
         keys[tid] = x;
         __syncthreads();
-    } else
-    for (int k = 2; k <= N; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = tid; i < N; i += NT) {
-                int ixj = i ^ j;
-                if (ixj > i) {
-                    unsigned x = keys[i], y = keys[ixj];
-                    bool up = (i & k) == 0;
-                    if ((x > y) == up) { keys[i] = y; keys[ixj] = x; }
-                }
-            }
-            __syncthreads();
-        }
     }
+    else if (N == 2 * NT) bitonic_sort_in_registers<NT, 2>(keys, tid);
+    else if (N == 4 * NT) bitonic_sort_in_registers<NT, 4>(keys, tid);
+    else if (N == 8 * NT) bitonic_sort_in_registers<NT, 8>(keys, tid);
+    else if (EB_MAX >= 16 * NT && N == 16 * NT) bitonic_sort_in_registers<NT, (EB_MAX >= 16 * NT ? 16 : 1)>(keys, tid);
+    else lds_bitonic_sort<NT>(keys, N);
     constexpr unsigned POS_MASK = (1u << KEY_POS_BITS) - 1u;
 
     if (role < 2) {
@@ -1766,6 +1817,7 @@ struct CombArgs {
     int tile_w;                  // 0: the row image holds the whole row; else its width in floats (a multiple of 32), see finish_row
     int direct_only;             // beside fbw_flat: only the sequences that kernel leaves to this one (flat_direct)
     int small_elsewhere = 0;     // the sequences of comb_small() are written by the SMALL instance of this kernel, launched beside this one
+    int pad_rows = 0;            // the general instance also writes the rows of frames >= seq_len (no fbw_padfill in this call)
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1974,7 +2026,17 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
     int b, y;
     strip_index(a.B, &b, &y);
     const SeqMeta m = a.meta[b];
-    if (m.L == 0) return;                                      // fbw_padfill has written every row
+    if (!SMALL && a.pad_rows) {
+        // Stage after stage there is nothing for fbw_padfill to run beside: its rows -- frames >= seq_len, for
+        // this workgroup those among the eight frames at its own position in the sequence -- are written here,
+        // one launch less in front of the recursion.
+        const float hole = NEGLOG ? INF_F : 0.f;
+        for (int t = max(y * TC, m.L); t < min(a.T, y * TC + TC); t++) {
+            stream_const_row(a.out + t * a.ost_t + b * a.ost_b, a.F, hole);
+            if (tid == 0) a.sum_output[(size_t)t * a.B + b] = 0.f;
+        }
+    }
+    if (m.L == 0) return;                                      // rows of frames >= seq_len: above, or by fbw_padfill
     if (a.direct_only && !flat_direct(m)) return;
     if (SMALL ? !comb_small(m) : (a.small_elsewhere && comb_small(m))) return;
     const int T = a.T, B = a.B, F = a.F;
@@ -2976,7 +3038,10 @@ size_t prep_lds_bytes(int F) { return (size_t)(EB_MAX + PREP_AUX_WORDS) * 4 + (F
 // would need a second round of them take 512-thread workgroups, four to a unit.
 void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
     const size_t lds = prep_lds_bytes(pa.F);
-    if (3 * pa.B > 2 * P.n_cu) hipLaunchKernelGGL(fbw_prepare<512>, dim3(3, pa.B), dim3(512), lds, s, pa);
+    // 512 threads: four workgroups per compute unit for large batches (one round instead of two), and for sequences of up
+    // to 512 edges on average, which have no work for more (fewer waves at every barrier: 50 x 2 x 10 0.058 -> 0.052 ms per
+    // call, 500 x 32 x 264 0.178 -> 0.173; 750 edges per sequence: no difference; 256 threads: slower from 380 edges on)
+    if (3 * pa.B > 2 * P.n_cu || (long long)pa.E <= 512LL * pa.B) hipLaunchKernelGGL(fbw_prepare<512>, dim3(3, pa.B), dim3(512), lds, s, pa);
     else hipLaunchKernelGGL(fbw_prepare<1024>, dim3(3, pa.B), dim3(1024), lds, s, pa);
 }
 
@@ -3103,6 +3168,7 @@ size_t comb_lds_bytes(int F) { return (size_t)(((F + 32 + 3) >> 2) * 16) + (size
 constexpr int COMB_TILE_W = 12288;     // floats of a row that go through LDS at a time when the row does not fit: three workgroups per unit
 
 // schedule: -1 by problem size, 0 single stream, 1 overlapped; I6FBW_OVERLAP=0/1 sets the initial value
+std::atomic<int> g_all_frames_default{0};      // i6fbw_set_band(0), kept for callers of earlier versions: every call as with I6FBW_IN_ALL_FRAMES
 std::atomic<int> g_overlap_mode{[] {
     const char* e = getenv("I6FBW_OVERLAP");
     return e ? (e[0] == '0' ? 0 : 1) : -1;
@@ -3221,6 +3287,7 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     if (E > 0 && (!edges || !weights)) return I6FBW_ERR_INVALID_ARGUMENT;
     if (out_mode != I6FBW_OUT_NEG_LOG && out_mode != I6FBW_OUT_PROB && out_mode != I6FBW_OUT_NEG_PROB) return I6FBW_ERR_INVALID_ARGUMENT;
     if (input_flags & ~(I6FBW_IN_LOG_PROBS | I6FBW_IN_ALL_FRAMES)) return I6FBW_ERR_INVALID_ARGUMENT;
+    input_flags |= g_all_frames_default.load();
     if (out_stride_t < 0 || out_stride_b < 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (((uintptr_t)workspace & 255) != 0) return I6FBW_ERR_INVALID_ARGUMENT;
     if (B > 65535 || (T + TC - 1) / TC > 65535) return I6FBW_ERR_INVALID_ARGUMENT;   // grid limits
@@ -3408,9 +3475,10 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
         int rc = launch_recursion(); if (rc != I6FBW_OK) return rc;
     }
     // (with the flat writer, the row writer for the sequences fbw_flat leaves out is started below, behind the gather)
-    if (!flat) {
+    ca.pad_rows = (!flat && !overlap) ? 1 : 0;
+    if (!flat && overlap) {
         // Rows of frames beyond seq_len depend on seq_lens only: written beside the preparation, which
-        // leaves the memory system idle.
+        // leaves the memory system idle.  (Stage after stage the row writer takes them, see pad_rows.)
         StageTimer tm(4, sP, timed);
         hipLaunchKernelGGL(fbw_padfill, p_grid, dim3(COMB_THREADS), 0, sP, seq_lens, T, B, F, out_mode, out, (long long)out_stride_t,
                            (long long)out_stride_b, sum_output);
@@ -3591,6 +3659,8 @@ int i6fbw_set_spin_limit(int polls) {
 
 void i6fbw_set_dense_writer(int mode) { g_writer_mode = mode < 0 ? -1 : (mode ? 1 : 0); }
 int i6fbw_last_dense_writer(void) { return g_last_writer.load(); }
+
+void i6fbw_set_band(int on) { g_all_frames_default = on ? 0 : I6FBW_IN_ALL_FRAMES; }
 
 void i6fbw_set_overlap(int mode) {
     std::lock_guard<std::mutex> lock(g_mutex);

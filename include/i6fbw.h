@@ -229,6 +229,14 @@ int i6fbw_viterbi(const float* am_scores, int64_t am_stride_t, int64_t am_stride
 void i6fbw_set_overlap(int mode);
 
 /*
+ * DEPRECATED, kept so that code written against earlier versions of this header still builds and behaves:
+ * i6fbw_set_band(0) makes every later call of the process run as if it had been given I6FBW_IN_ALL_FRAMES,
+ * i6fbw_set_band(1) (the default) ends that.  New code passes the flag to the one call that needs it
+ * (i6fbw_run_strided).  No counterpart in the reference.
+ */
+void i6fbw_set_band(int on);
+
+/*
  * TEST HOOK, not for production code.  Kernels of the overlapped schedule that wait for another kernel
  * of the same call poll at most `polls` times (default 2^20, restored by polls <= 0) before they give up:
  * the call then reports I6FBW_ERR_TIMEOUT and the rows that could not be computed hold NaN.  It exists so

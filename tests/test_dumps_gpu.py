@@ -115,6 +115,36 @@ def test_dump_every_and_defaults(in_tmp):
     assert not glob.glob("alignment.dump.*")
 
 
+def test_process_wide_switch_of_earlier_versions_still_works(in_tmp):
+    """i6fbw_set_band(0), the process-wide switch that the per-call flag I6FBW_IN_ALL_FRAMES replaced, is still
+    exported for code written against earlier versions of the header: a run under it leaves the same forward rows
+    (the same alignment dump) as a run with the flag, and i6fbw_set_band(1) ends it."""
+    from i6_native_ops_amd import cabi
+    from i6_native_ops_amd.fbw.workloads import make_workload
+    from tests.gpu_util import DeviceProblem
+    wl = make_workload("tiny")
+    P = DeviceProblem(wl.am_scores, wl.edges, wl.weights, wl.start_end_states, wl.seq_lens, wl.n_states)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def dump(idx, **kw):
+        out, loss = P.run(cabi.OUT_NEG_LOG, **kw)
+        cabi.dump_alignment(P.ws.data_ptr(), P.T, P.B, P.E, P.start_end.data_ptr(), P.start_end.stride(0), 1e30, idx, ".", stream)
+        return [open(f"alignment.dump.{idx}.{b}").read() for b in range(wl.B)], out.clone(), loss.clone()
+
+    with_flag, out1, loss1 = dump(1, input_flags=cabi.IN_ALL_FRAMES)
+    lib = cabi.load()
+    lib.i6fbw_set_band(0)
+    try:
+        with_switch, out2, loss2 = dump(2)
+    finally:
+        lib.i6fbw_set_band(1)
+    banded, out3, loss3 = dump(3)
+    assert with_switch == with_flag
+    assert torch.equal(out1, out2) and torch.equal(loss1, loss2)
+    assert banded != with_flag                    # states that cannot reach the end have no score inside the band
+    torch.testing.assert_close(out3, out1, rtol=1e-6, atol=1e-6)
+
+
 def test_dump_through_the_c_abi(in_tmp, oracle):
     """Two sequences with different lengths straight through i6fbw_dump_*: occupancies of a frame sum to 1,
     the target file lists exactly the finite entries of out."""

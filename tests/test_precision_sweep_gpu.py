@@ -204,6 +204,31 @@ def test_tight_chains_under_arbitrary_state_ids(oracle, companions, shuffle):
     assert worst <= PERMUTED_IDS_BOUND
 
 
+def test_tight_chain_whose_permuted_ids_span_less_than_twice_its_edges(oracle):
+    """One chain of 1021 states over 1100 frames beside eight small sequences, ids permuted over the whole batch: the
+    ids of the chain then span about 3500 values -- too few for the sequence to count as one with spread ids (more
+    than 2 * edges + 2), too many for the numbering along the automaton, which holds 2048 states, to take the span
+    for the number of states (7.9e-5 in the random runs before such a sequence had its ids ranked first)."""
+    from tests.helpers import spread_state_ids
+    from tests.test_flat_writer_gpu import merge
+    T = 1100
+    parts = [make_workload("cart", seed=4242, T=T, B=8, F=600, n_labels=(5, 11), shuffle_edges=False),
+             make_workload("cart", seed=955309586, T=T, B=1, F=600, n_labels=(340, 340), shuffle_edges=False)]
+    for p in parts:
+        p.seq_lens[:] = T
+    am, edges, weights, se, lens, n_states = merge(parts)
+    edges, se, n_states = spread_state_ids(edges, se, n_states, "permute", seed=3)
+    big = edges[3] == 8
+    span = int(max(edges[0, big].max(), edges[1, big].max()) - min(edges[0, big].min(), edges[1, big].min())) + 1
+    assert 2048 < span <= 2 * int(big.sum()) + 2, span             # the case this test is about
+    failures, worst = [], 0.0
+    for overlap in (0, 1):
+        worst = max(worst, check(oracle, _Args(am, edges, weights, se, lens, n_states), overlap,
+                                 f"one chain of 1021 states, ids permuted over a batch of nine, overlap={overlap}", failures))
+    assert not failures, failures
+    assert worst <= PERMUTED_IDS_BOUND
+
+
 def test_large_batch_of_tight_monophone_automata(oracle):
     """140 monophone automata of 200 to 400 states over 320 to 400 frames, many of them with barely more frames than
     states, in one batch: the recursion instance of which two workgroups share a compute unit, whose sequences of
