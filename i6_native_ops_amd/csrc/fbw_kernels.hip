@@ -68,6 +68,8 @@ constexpr int RENORM = 8;             // frames between renormalisations of the 
 constexpr int COMB_THREADS = 256;
 constexpr int COMB_JD = D_MAX / COMB_THREADS;
 constexpr int COMB_XS = 1024;         // edge scores staged in LDS per pass of the combine kernel
+constexpr int COMB_BATCH = 4;         // frames the row writer takes together for sequences of up to COMB_BATCH_EDGES edges (rows of up to COMB_BATCH_F floats)
+constexpr int COMB_BATCH_EDGES = 512, COMB_BATCH_F = 1024;
 constexpr int COMB_MID_EDGES = 4096;  // up to here a combine workgroup keeps the edges of its sequence in registers ...
 constexpr int COMB_MID_SLOTS = 2048;  // ... and the distinct emissions of the sequence spread over its threads' registers
 #ifndef I6_FLOAT_FRAMES
@@ -1824,6 +1826,7 @@ struct CombArgs {
     int direct_only;             // beside fbw_flat: only the sequences that kernel leaves to this one (flat_direct)
     int small_elsewhere = 0;     // the sequences of comb_small() are written by the SMALL instance of this kernel, launched beside this one
     int pad_rows = 0;            // the general instance also writes the rows of frames >= seq_len (no fbw_padfill in this call)
+    int batch_frames = 0;        // SMALL instance: the LDS of the launch holds COMB_BATCH row images and staging areas (comb_batch_lds_bytes)
 };
 
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -1949,6 +1952,34 @@ __device__ __forceinline__ float slot_sum(const float* xs, const int c0, const i
         if (lane == src) s = p;
     }
     return s;
+}
+
+// The same for MF frames whose staged values lie `stride` apart: the frames' LDS reads are independent of each other, so
+// a lane's short range costs one read latency per entry for all of them.  Frame by frame the additions are slot_sum's.
+template <int MF>
+__device__ __forceinline__ void slot_sum_frames(const float* xs, const int stride, const int c0, const int c1, float (&s)[MF]) {
+    const int lane = threadIdx.x & 63;
+    const bool is_long = c1 - c0 > LONG_SLOT;
+#pragma unroll
+    for (int f = 0; f < MF; f++) s[f] = 0.f;
+    if (!is_long)
+        for (int i = c0; i < c1; i++) {
+#pragma unroll
+            for (int f = 0; f < MF; f++) s[f] += xs[f * stride + i];
+        }
+    unsigned long long todo = __ballot(is_long);
+    while (todo) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int b0 = __builtin_amdgcn_readlane(c0, src), b1 = __builtin_amdgcn_readlane(c1, src);
+#pragma unroll
+        for (int f = 0; f < MF; f++) {
+            float p = 0.f;
+            for (int q = b0 + lane; q < b1; q += 64) p += xs[f * stride + q];
+            p = lane63(wave_sum_dpp(p));
+            if (lane == src) s[f] = p;
+        }
+    }
 }
 
 // The same in log space, for the -log output (NEGLOG instances of the kernels below): xs holds the raw
@@ -2184,7 +2215,126 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
         stream_image_row(orow, F, lds4, image);
     };
 
-    if (SMALL || (nE <= COMB_XS && D <= 2 * COMB_THREADS)) {
+    if (SMALL && !NEGLOG && a.batch_frames && nE <= COMB_BATCH_EDGES) {
+        // Small sequences, short rows: COMB_BATCH frames at a time.  Every step of a frame -- minimum, staging,
+        // per-emission sums, total, row image, row -- is an LDS round trip and a barrier for four waves, about 400
+        // cycles each whatever the amount of work, and a frame has ten of them (1.8 us per frame for 30 edges as
+        // for 400); taken for four frames together they cost the same once.  Same arithmetic in the same order as
+        // the path below, frame by frame, hence the same bits.  (50 x 2 x 10: 0.052 -> 0.047 ms per call; 500 x 32 x 264:
+        // row writer 44 -> 38 us.)
+        constexpr int MF = COMB_BATCH, JE = COMB_BATCH_EDGES / COMB_THREADS, JS = 2;
+        __shared__ float red4[2][MF][COMB_THREADS / 64];
+        float* xsb = image + (size_t)MF * 4 * F4;                 // MF x COMB_BATCH_EDGES staged probabilities
+        for (int i = F4 + tid; i < MF * F4; i += COMB_THREADS) lds4[i] = (float4a){hole, hole, hole, hole};      // (the first image: above)
+        unsigned efr[JE], eto[JE], esl[JE];
+        float ew[JE];
+#pragma unroll
+        for (int j = 0; j < JE; j++) {
+            const int i = tid + j * COMB_THREADS;
+            uint4 r = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
+            if (i < nE) r = crec[i];
+            efr[j] = r.x & 0xFFFFu; eto[j] = r.x >> 16; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
+        }
+        int c0[JS], c1[JS], em[JS];
+#pragma unroll
+        for (int js = 0; js < JS; js++) {
+            const int d = tid + js * COMB_THREADS;
+            c0[js] = c1[js] = em[js] = 0;
+            if (d < D) { c0[js] = cb[d]; c1[js] = cb[d + 1]; em[js] = de[d]; }
+        }
+        const int wave = tid >> 6, lane = tid & 63;
+        for (int tb = t0; tb < tv; tb += MF) {
+            const int nf = min(MF, tv - tb);
+            // operands of all frames of the batch in one round trip (frames past the end: the last one once more, unused)
+            float x[MF][JE], lmin[MF];
+            // the row offsets: lane 2f has the alpha row's of frame f, lane 2f+1 the beta row's
+            const double voff = tid < 2 * nf ? load_x<SYNC>(((tid & 1) ? offB : offA) + tb + (tid >> 1)) : 0.0;
+            {
+                float va[MF][JE], vb[MF][JE], vg[MF][JE];
+#pragma unroll
+                for (int f = 0; f < MF; f++) {
+                    const int t = min(tb + f, tv - 1);
+                    const float* arow = abase + (size_t)t * SP;
+                    const float* brow = bbase + (size_t)t * SP;
+                    const float* grow = gbase + (size_t)t * DP;
+#pragma unroll
+                    for (int j = 0; j < JE; j++) {
+                        va[f][j] = load_x<SYNC>(arow + efr[j]); vb[f][j] = load_x<SYNC>(brow + eto[j]); vg[f][j] = load_x<SYNC>(grow + esl[j]);
+                    }
+                }
+#pragma unroll
+                for (int f = 0; f < MF; f++) {
+                    lmin[f] = INF_F;
+#pragma unroll
+                    for (int j = 0; j < JE; j++) { x[f][j] = (va[f][j] + ew[j]) + (vg[f][j] + vb[f][j]); lmin[f] = fminf(lmin[f], x[f][j]); }
+                }
+            }
+            float mn[MF];
+#pragma unroll
+            for (int f = 0; f < MF; f++) {
+                const float v = wave_min_dpp(lmin[f]);
+                if (lane == 63) red4[0][f][wave] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int f = 0; f < MF; f++) {
+                mn[f] = fminf(fminf(red4[0][f][0], red4[0][f][1]), fminf(red4[0][f][2], red4[0][f][3]));
+#pragma unroll
+                for (int j = 0; j < JE; j++) xsb[f * COMB_BATCH_EDGES + tid + j * COMB_THREADS] = mn[f] == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn[f] - x[f][j]);
+            }
+            __syncthreads();
+            // per-emission sums in fixed (input) order, then the frame normalisers
+            float sd[MF][JS], tot[MF];
+#pragma unroll
+            for (int js = 0; js < JS; js++) {
+                float s4[MF];
+                slot_sum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], s4);
+#pragma unroll
+                for (int f = 0; f < MF; f++) sd[f][js] = s4[f];
+            }
+#pragma unroll
+            for (int f = 0; f < MF; f++) {
+                float part = 0.f;
+#pragma unroll
+                for (int js = 0; js < JS; js++) part += sd[f][js];
+                const float v = wave_sum_dpp(part);
+                if (lane == 63) red4[1][f][wave] = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int f = 0; f < MF; f++) tot[f] = (red4[1][f][0] + red4[1][f][1]) + (red4[1][f][2] + red4[1][f][3]);
+            // loss, image positions, rows
+            int shf[MF];
+#pragma unroll
+            for (int f = 0; f < MF; f++) {
+                const double offs = __shfl(voff, 2 * f) + __shfl(voff, 2 * f + 1);
+                shf[f] = 0;
+                if (f < nf) {
+                    const int t = tb + f;
+                    const bool dead = mn[f] == INF_F;
+                    const float logtot = __builtin_amdgcn_logf(tot[f]);
+                    if (tid == 0) a.sum_output[(size_t)t * B + b] = dead ? 0.f : (float)(((double)(mn[f] - logtot) + offs) * (double)LN2);
+                    const float inv = dead ? 0.f : psign / tot[f];
+                    shf[f] = row_misalign(a.out + t * a.ost_t + b * a.ost_b);
+#pragma unroll
+                    for (int js = 0; js < JS; js++)
+                        if (tid + js * COMB_THREADS < D) image[(size_t)f * 4 * F4 + shf[f] + em[js]] = sd[f][js] * inv;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int f = 0; f < MF; f++)
+                if (f < nf) stream_image_row(a.out + (tb + f) * a.ost_t + b * a.ost_b, F, lds4 + (size_t)f * F4, image + (size_t)f * 4 * F4);
+            __syncthreads();
+#pragma unroll
+            for (int f = 0; f < MF; f++)
+                if (f < nf) {
+#pragma unroll
+                    for (int js = 0; js < JS; js++)
+                        if (tid + js * COMB_THREADS < D) image[(size_t)f * 4 * F4 + shf[f] + em[js]] = hole;
+                }
+        }
+    } else if (SMALL || (nE <= COMB_XS && D <= 2 * COMB_THREADS)) {
         // fast path: this thread's edges and slots stay in registers for the whole strip, and
         // the operands of the next frame are fetched while the current one is processed
         constexpr int JE = COMB_XS / COMB_THREADS, JS = 2;
@@ -3054,11 +3204,16 @@ void launch_prepare(const Pipeline& P, const PrepArgs& pa, hipStream_t s) {
 // The dense writers, in the instance for the output mode (NEGLOG: the -log output, summed in log space)
 // (the row writer proper: first the instance for small sequences -- most batches are nothing else -- then the general
 // one for the rest; rows too long for the LDS image, and the sequences fbw_flat leaves over, are the general one's alone)
+// (LDS of the small-sequence instance where it takes COMB_BATCH frames together: that many row images and staging areas)
+size_t comb_batch_lds_bytes(int F) { return (size_t)COMB_BATCH * ((size_t)(((F + 32 + 3) >> 2) * 16) + (size_t)COMB_BATCH_EDGES * 4); }
 template <bool SYNC>
 void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStream_t s, CombArgs ca) {
     if (!ca.direct_only && !ca.tile_w) {
-        if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, true>), grid, dim3(COMB_THREADS), lds, s, ca);
-        else hipLaunchKernelGGL((fbw_combine<SYNC, false, true>), grid, dim3(COMB_THREADS), lds, s, ca);
+        CombArgs cs = ca;
+        size_t lds_s = lds;
+        if (!neglog && ca.F <= COMB_BATCH_F) { cs.batch_frames = 1; lds_s = std::max(lds, comb_batch_lds_bytes(ca.F)); }
+        if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
+        else hipLaunchKernelGGL((fbw_combine<SYNC, false, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
         ca.small_elsewhere = 1;
     }
     if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, false>), grid, dim3(COMB_THREADS), lds, s, ca);
