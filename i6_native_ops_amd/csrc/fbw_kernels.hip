@@ -2014,6 +2014,42 @@ __device__ __forceinline__ LogSum slot_logsum(const float* xs, const int c0, con
     }
     return r;
 }
+// slot_logsum for MF frames whose staged scores lie `stride` apart (see slot_sum_frames); frame by frame slot_logsum's arithmetic
+template <int MF>
+__device__ __forceinline__ void slot_logsum_frames(const float* xs, const int stride, const int c0, const int c1, LogSum (&r)[MF]) {
+    const int lane = threadIdx.x & 63;
+    const bool is_long = c1 - c0 > LONG_SLOT;
+#pragma unroll
+    for (int f = 0; f < MF; f++) { r[f].mn = INF_F; r[f].sum = 0.f; }
+    if (!is_long) {
+        for (int i = c0; i < c1; i++) {
+#pragma unroll
+            for (int f = 0; f < MF; f++) r[f].mn = fminf(r[f].mn, xs[f * stride + i]);
+        }
+        for (int i = c0; i < c1; i++) {
+#pragma unroll
+            for (int f = 0; f < MF; f++)
+                if (r[f].mn < INF_F) r[f].sum += __builtin_amdgcn_exp2f(r[f].mn - xs[f * stride + i]);
+        }
+    }
+    unsigned long long todo = __ballot(is_long);
+    while (todo) {
+        const int src = __ffsll((long long)todo) - 1;
+        todo &= todo - 1;
+        const int b0 = __builtin_amdgcn_readlane(c0, src), b1 = __builtin_amdgcn_readlane(c1, src);
+#pragma unroll
+        for (int f = 0; f < MF; f++) {
+            float pm = INF_F;
+            for (int q = b0 + lane; q < b1; q += 64) pm = fminf(pm, xs[f * stride + q]);
+            pm = lane63(wave_min_dpp(pm));
+            float p = 0.f;
+            if (pm < INF_F)
+                for (int q = b0 + lane; q < b1; q += 64) p += __builtin_amdgcn_exp2f(pm - xs[f * stride + q]);
+            p = lane63(wave_sum_dpp(p));
+            if (lane == src) { r[f].mn = pm; r[f].sum = p; }
+        }
+    }
+}
 // a (+)= b for two pieces of one slot (edges staged in passes).  A slot that lies in one piece keeps the
 // bits of that piece.
 __device__ __forceinline__ void logsum_merge(LogSum& a, const LogSum b) {
@@ -2215,13 +2251,13 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
         stream_image_row(orow, F, lds4, image);
     };
 
-    if (SMALL && !NEGLOG && a.batch_frames && nE <= COMB_BATCH_EDGES) {
+    if (SMALL && a.batch_frames && nE <= COMB_BATCH_EDGES) {
         // Small sequences, short rows: COMB_BATCH frames at a time.  Every step of a frame -- minimum, staging,
         // per-emission sums, total, row image, row -- is an LDS round trip and a barrier for four waves, about 400
         // cycles each whatever the amount of work, and a frame has ten of them (1.8 us per frame for 30 edges as
         // for 400); taken for four frames together they cost the same once.  Same arithmetic in the same order as
-        // the path below, frame by frame, hence the same bits.  (50 x 2 x 10: 0.052 -> 0.047 ms per call; 500 x 32 x 264:
-        // row writer 44 -> 38 us.)
+        // the path below, frame by frame, hence the same bits, in the -log instance too.  (50 x 2 x 10: 0.052 -> 0.047 ms
+        // per call; 500 x 32 x 264: row writer 44 -> 38 us.)
         constexpr int MF = COMB_BATCH, JE = COMB_BATCH_EDGES / COMB_THREADS, JS = 2;
         __shared__ float red4[2][MF][COMB_THREADS / 64];
         float* xsb = image + (size_t)MF * 4 * F4;                 // MF x COMB_BATCH_EDGES staged probabilities
@@ -2276,33 +2312,54 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
                 if (lane == 63) red4[0][f][wave] = v;
             }
             __syncthreads();
+            // staged per frame: the probabilities relative to the frame minimum (-log instance: the raw scores, and
+            // the frame normaliser is the sum over the edges, in edge order per thread, as in the path below)
+            float part[MF];
 #pragma unroll
             for (int f = 0; f < MF; f++) {
                 mn[f] = fminf(fminf(red4[0][f][0], red4[0][f][1]), fminf(red4[0][f][2], red4[0][f][3]));
+                part[f] = 0.f;
 #pragma unroll
-                for (int j = 0; j < JE; j++) xsb[f * COMB_BATCH_EDGES + tid + j * COMB_THREADS] = mn[f] == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn[f] - x[f][j]);
+                for (int j = 0; j < JE; j++) {
+                    const float p = mn[f] == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn[f] - x[f][j]);
+                    if (NEGLOG) part[f] += p;
+                    xsb[f * COMB_BATCH_EDGES + tid + j * COMB_THREADS] = NEGLOG ? x[f][j] : p;
+                }
             }
-            __syncthreads();
-            // per-emission sums in fixed (input) order, then the frame normalisers
-            float sd[MF][JS], tot[MF];
+            // per-emission sums in fixed (input) order and the frame normalisers
+            float val[MF][JS], tot[MF];
+            if (!NEGLOG) {
+                __syncthreads();
 #pragma unroll
-            for (int js = 0; js < JS; js++) {
-                float s4[MF];
-                slot_sum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], s4);
+                for (int js = 0; js < JS; js++) {
+                    float s4[MF];
+                    slot_sum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], s4);
 #pragma unroll
-                for (int f = 0; f < MF; f++) sd[f][js] = s4[f];
+                    for (int f = 0; f < MF; f++) val[f][js] = s4[f];
+                }
+#pragma unroll
+                for (int f = 0; f < MF; f++)
+#pragma unroll
+                    for (int js = 0; js < JS; js++) part[f] += val[f][js];
             }
 #pragma unroll
             for (int f = 0; f < MF; f++) {
-                float part = 0.f;
-#pragma unroll
-                for (int js = 0; js < JS; js++) part += sd[f][js];
-                const float v = wave_sum_dpp(part);
+                const float v = wave_sum_dpp(part[f]);
                 if (lane == 63) red4[1][f][wave] = v;
             }
-            __syncthreads();
+            __syncthreads();              // (-log instance: also publishes the staged scores)
 #pragma unroll
             for (int f = 0; f < MF; f++) tot[f] = (red4[1][f][0] + red4[1][f][1]) + (red4[1][f][2] + red4[1][f][3]);
+            if (NEGLOG) {
+#pragma unroll
+                for (int js = 0; js < JS; js++) {
+                    LogSum l4[MF];
+                    slot_logsum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], l4);
+#pragma unroll
+                    for (int f = 0; f < MF; f++)
+                        val[f][js] = mn[f] == INF_F ? INF_F : neg_log_value(l4[f], mn[f], __builtin_amdgcn_logf(tot[f]));
+                }
+            }
             // loss, image positions, rows
             int shf[MF];
 #pragma unroll
@@ -2318,7 +2375,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
                     shf[f] = row_misalign(a.out + t * a.ost_t + b * a.ost_b);
 #pragma unroll
                     for (int js = 0; js < JS; js++)
-                        if (tid + js * COMB_THREADS < D) image[(size_t)f * 4 * F4 + shf[f] + em[js]] = sd[f][js] * inv;
+                        if (tid + js * COMB_THREADS < D) image[(size_t)f * 4 * F4 + shf[f] + em[js]] = NEGLOG ? val[f][js] : val[f][js] * inv;
                 }
             }
             __syncthreads();
@@ -3211,7 +3268,7 @@ void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStr
     if (!ca.direct_only && !ca.tile_w) {
         CombArgs cs = ca;
         size_t lds_s = lds;
-        if (!neglog && ca.F <= COMB_BATCH_F) { cs.batch_frames = 1; lds_s = std::max(lds, comb_batch_lds_bytes(ca.F)); }
+        if (ca.F <= COMB_BATCH_F) { cs.batch_frames = 1; lds_s = std::max(lds, comb_batch_lds_bytes(ca.F)); }
         if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
         else hipLaunchKernelGGL((fbw_combine<SYNC, false, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
         ca.small_elsewhere = 1;

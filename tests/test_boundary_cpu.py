@@ -180,8 +180,8 @@ def test_kernels_stay_within_their_register_budgets():
         if small:
             # the instance for sequences of up to 1024 edges: six workgroups per compute unit.  Its scratch: values that
             # do not change over a strip of frames, stored once in front of the frame loop and read back once per
-            # batch of four frames (posterior modes) or per frame (-log) -- nothing per edge
-            assert r["vgprs"] <= 80 and r["occupancy"] >= 6 and r["scratch"] <= (8 if neglog else 40), (name, r)
+            # batch of four frames -- nothing per edge or per frame
+            assert r["vgprs"] <= 80 and r["occupancy"] >= 6 and r["scratch"] <= (72 if neglog else 40), (name, r)
         elif neglog:
             # the instance for the -log output: a few reloads per frame on its paths for sequences of more than 1024
             # edges (with two waves per SIMD it needs none and is slower)
