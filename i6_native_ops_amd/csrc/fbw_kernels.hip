@@ -73,7 +73,8 @@ constexpr int COMB_BATCH_EDGES = 512, COMB_BATCH_F = 1024;
 constexpr int COMB_MID_EDGES = 4096;  // up to here a combine workgroup keeps the edges of its sequence in registers ...
 constexpr int COMB_MID_SLOTS = 2048;  // ... and the distinct emissions of the sequence spread over its threads' registers
 #ifndef I6_FLOAT_FRAMES
-#define I6_FLOAT_FRAMES 512           // sequences with more frames keep their state vectors in double
+#define I6_FLOAT_FRAMES 256           // sequences with more frames keep their state vectors in double (with one or two states per thread double
+                                      // costs these instances nothing measurable; 177 states over 400 frames in float: 7.1e-5, in double 9.8e-6)
 #endif
 constexpr int REC_THREADS = 512;      // compute threads of a recursion workgroup
 constexpr int REC_LOADERS = 1;        // loader waves beside them
@@ -1741,9 +1742,10 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // 1055 frames 1.4e-4; 20 000 frames through 100 states 3e-4).  Up to 256 states -- one wave per
     // SIMD, bound by latency more than by arithmetic -- double costs 7 % of the recursion and is used
     // for sequences with fewer than four frames per state; beyond that it costs 15-20 % and is kept for
-    // sequences with fewer than five frames for every three states.  More than 1024 frames: always
-    // (whatever the shape of the automaton, float adds up to about 1e-4 over 2000 frames: CTC automata of
-    // 200 labels over 2000 frames 9.7e-5, of 400 labels over 2600 frames 8e-5).
+    // sequences with fewer than five frames for every three states.  More than I6_FLOAT_FRAMES frames: always
+    // (whatever the shape of the automaton, float adds up from frame to frame: CTC automata of 200 labels over
+    // 2000 frames 9.7e-5, 177 states over 400 frames 7.1e-5; the sequences this rule alone catches have at most
+    // three states for every five frames, i.e. few states per thread, where double costs next to nothing).
     // The dense instance has room in LDS for the small sequences only (and is used for at most 4096
     // frames): batches of more than 128 CTC automata of 110-150 labels over 760-900 frames came out at
     // 8.7e-5 to 9.3e-5 in float.
