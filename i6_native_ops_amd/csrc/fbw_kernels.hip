@@ -3647,8 +3647,13 @@ int run_impl(const float* am, int64_t am_stride_t, int64_t am_stride_b, int inpu
     // The preparation's workgroups can do the gate's wait themselves (one kernel less in front of the gather)
     // where they cannot be in the recursion's way: a preparation workgroup and a recursion workgroup do not
     // share a compute unit, the order in which the two kernels are placed is not ours, and a preparation
-    // workgroup that waits keeps its unit -- so only if both grids fit with a unit per workgroup.
-    const bool gate_in_prepare = early && 5 * B <= P.n_cu;
+    // workgroup that waits keeps its unit -- so only if both grids fit with a unit per workgroup.  Workgroups are
+    // dealt out to the device's XCDs in turn, so the units have to be there XCD by XCD, each with its share of either
+    // grid rounded up: 51 sequences are 20 + 13 workgroups for the first XCD's 32 units -- 5 B <= 256, and the
+    // thirteenth recursion workgroup waited for a unit until the preparation's waits ran out.  (Four units per XCD
+    // are left over for whatever else is on the machine.)
+    constexpr int XCDS = 8;
+    const bool gate_in_prepare = early && (3 * B + XCDS - 1) / XCDS + (2 * B + XCDS - 1) / XCDS <= P.n_cu / XCDS - 4;
     pa.gate_need = gate_in_prepare ? 2 * B : 0;
     auto launch_recursion = [&]() -> int {
         { StageTimer tm(2, sR, timed); if (dense) hipLaunchKernelGGL(fbw_recurse_dense<true>, dim3(2 * B), dim3(REC_BLOCK_DENSE), sizeof(float) * REC_LDS_FLOATS_F32, sR, ra);

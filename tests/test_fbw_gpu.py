@@ -89,6 +89,9 @@ def test_tightly_constrained_alignment(oracle):
     ("cart", dict(T=40, B=2, F=38000, n_labels=(8, 12))),     # the largest row images that fit into LDS
     ("ctc", dict(T=40, B=8, F=50)),
     ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
+    ("cart", dict(T=60, B=44, F=300, n_labels=(5, 9))),      # the largest batch whose preparation holds the gather back itself: five workgroups per sequence, a unit each
+    ("cart", dict(T=60, B=45, F=300, n_labels=(5, 9))),      # one more: a one-wave kernel does it
+    ("ctc", dict(T=130, B=51, F=40, n_labels=(60, 80))),     # 5 B = 255 units in all, but 33 workgroups for the first XCD's 32 (this batch ran into the bound of its waits)
     ("cart", dict(T=60, B=64, F=300, n_labels=(5, 9))),      # a recursion workgroup on half of the compute units: started beside the preparation
     ("cart", dict(T=60, B=65, F=300, n_labels=(5, 9))),      # one more: started behind it
     ("cart", dict(T=60, B=128, F=300, n_labels=(5, 9))),     # one on every compute unit: gather and dense write must still find room
