@@ -1751,12 +1751,12 @@ __device__ __forceinline__ void recurse_workgroup(const RecArgs& a, float* lds) 
     // 8.7e-5 to 9.3e-5 in float.
     const bool small_tight = cls == 1 && m.SP <= 256 && m.L < 4LL * m.S;
     const bool wide = !DENSE && (small_tight || 5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES);
-    // (there double costs half of the recursion time again, so only from 384 frames on, where the
-    // rounding of float has had time to add up -- but then for every sequence with one state per thread --
-    // and from 256 frames on for the tightly aligned ones: 140 monophone automata of 250-400 states over
-    // 320-400 frames came out at 8.7e-5 in float, 3.6e-5 in double; CTC automata of 40-120 states over 150-200
-    // frames are at 1.7e-5 in float and would pay 14 us per call)
-    if (DENSE && cls == 1 && (m.L >= 384 || (m.L >= 256 && 5LL * m.S > 3LL * m.L)) && (dir ? m.Kout : m.Kin) <= KMAX) {
+    // (there double costs 5-12 % of the recursion time, so only from 256 frames on, where the rounding of float has
+    // had time to add up -- but then for every sequence with one state per thread: 140 automata of up to 180 states
+    // over up to 400 frames came out at 6.5e-5 in float, 2.4e-5 in double; 140 monophone automata of 250-400 states
+    // over 320-400 frames at 8.7e-5 and 3.6e-5; CTC automata of 40-120 states over 150-200 frames are at 1.7e-5
+    // in float and would pay 14 us per call)
+    if (DENSE && cls == 1 && m.L >= I6_FLOAT_FRAMES && (dir ? m.Kout : m.Kin) <= KMAX) {
         double* st0 = (double*)stf;
         recurse_dispatch<SYNC, T_, double, true, false>(a, m, b, dir, cls, st0, st0 + (T_ + 16), amr[0], amr[1], wmin);
     } else if (DENSE && cls >= 2 && (5LL * m.S > 3LL * m.L || m.L > I6_FLOAT_FRAMES)) {

@@ -86,6 +86,7 @@ def test_shapes_next_to_the_precision_decisions(oracle, overlap):
 
 # more than 128 sequences: the instance with 448 compute threads of which two share a compute unit
 DENSE_CASES = [
+    ("ctc", 48, 255), ("ctc", 48, 256), ("cart", 40, 255), ("cart", 40, 256), ("cart", 59, 380),
     ("ctc", 48, 383), ("ctc", 48, 384), ("ctc", 48, 399), ("ctc", 100, 500), ("cart", 40, 383), ("cart", 40, 384),
     ("ctc", 60, 1024), ("ctc", 60, 1025), ("cart", 120, 1100),
     # more states than the instance has compute threads (several states per thread), short and long
