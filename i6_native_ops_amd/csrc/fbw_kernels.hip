@@ -2081,8 +2081,11 @@ __device__ __forceinline__ float neg_log_value(const LogSum s, const float mn, c
 // batch then run at the same time (monophone configuration: dense write 58 -> 42 us, call 0.194 -> 0.178 ms; four or six
 // workgroups per unit measure the same, eight need 64 registers and spill: 50 us).  The host launches it next to the
 // general instance, which leaves those sequences out (small_elsewhere).
-__device__ __forceinline__ bool comb_small(const SeqMeta& m) {
-    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= COMB_XS && m.D <= 2 * COMB_THREADS;
+// (with short rows -- batch: the launch has the LDS for several row images and a staging area of 2048 values -- also up to
+// 2048 edges: a single pass through the staging area and two slots per thread where the general instance takes passes of
+// 1024 edges with eight slots per thread and fetches sixteen edges per thread whatever their number)
+__device__ __forceinline__ bool comb_small(const SeqMeta& m, const int batch) {
+    return seq_error(m) == 0 && m.n_edges > 0 && m.L > 0 && m.n_edges <= (batch ? COMB_BATCH * COMB_BATCH_EDGES : COMB_XS) && m.D <= 2 * COMB_THREADS;
 }
 #ifndef I6_COMB_SMALL_OCC
 #define I6_COMB_SMALL_OCC 6
@@ -2113,7 +2116,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
     }
     if (m.L == 0) return;                                      // rows of frames >= seq_len: above, or by fbw_padfill
     if (a.direct_only && !flat_direct(m)) return;
-    if (SMALL ? !comb_small(m) : (a.small_elsewhere && comb_small(m))) return;
+    if (SMALL ? !comb_small(m, a.batch_frames) : (a.small_elsewhere && comb_small(m, a.batch_frames))) return;
     const int T = a.T, B = a.B, F = a.F;
     // strips of TC frames are handed out from the middle of the sequence outwards: that is where the
     // forward and the backward recursion meet, so those rows are complete first
@@ -2253,25 +2256,26 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
         stream_image_row(orow, F, lds4, image);
     };
 
-    if (SMALL && a.batch_frames && nE <= COMB_BATCH_EDGES) {
-        // Small sequences, short rows: COMB_BATCH frames at a time.  Every step of a frame -- minimum, staging,
-        // per-emission sums, total, row image, row -- is an LDS round trip and a barrier for four waves, about 400
-        // cycles each whatever the amount of work, and a frame has ten of them (1.8 us per frame for 30 edges as
-        // for 400); taken for four frames together they cost the same once.  Same arithmetic in the same order as
-        // the path below, frame by frame, hence the same bits, in the -log instance too.  (50 x 2 x 10: 0.052 -> 0.047 ms
-        // per call; 500 x 32 x 264: row writer 44 -> 38 us.)
-        constexpr int MF = COMB_BATCH, JE = COMB_BATCH_EDGES / COMB_THREADS, JS = 2;
-        __shared__ float red4[2][MF][COMB_THREADS / 64];
-        float* xsb = image + (size_t)MF * 4 * F4;                 // MF x COMB_BATCH_EDGES staged probabilities
+    // Small sequences, short rows: several frames at a time.  Every step of a frame -- minimum, staging, per-emission
+    // sums, total, row image, row -- is an LDS round trip and a barrier for four waves, about 400 cycles each whatever
+    // the amount of work, and a frame has ten of them (1.8 us per frame for 30 edges as for 400); taken for MF frames
+    // together they cost the same once.  Four frames with two edges per thread, two with four or one with eight, in the same
+    // registers and the same LDS.  Same arithmetic in the same order as the path below, frame by frame, hence the same
+    // bits, in the -log instance too.  (50 x 2 x 10: 0.052 -> 0.047 ms per call; 500 x 32 x 264: row writer 44 -> 38 us.)
+    __shared__ float red4[2][COMB_BATCH][COMB_THREADS / 64];
+    auto batched = [&](auto mf_, auto je_) {
+        constexpr int MF = decltype(mf_)::value, JE = decltype(je_)::value, JS = 2, XSTRIDE = JE * COMB_THREADS;
+        static_assert(MF <= COMB_BATCH && MF * XSTRIDE <= COMB_BATCH * COMB_BATCH_EDGES, "LDS of the launch: comb_batch_lds_bytes");
+        float* xsb = image + (size_t)MF * 4 * F4;                 // MF x XSTRIDE staged values
         for (int i = F4 + tid; i < MF * F4; i += COMB_THREADS) lds4[i] = (float4a){hole, hole, hole, hole};      // (the first image: above)
-        unsigned efr[JE], eto[JE], esl[JE];
+        unsigned eft[JE], esl[JE];           // source | target << 16, slot
         float ew[JE];
 #pragma unroll
         for (int j = 0; j < JE; j++) {
             const int i = tid + j * COMB_THREADS;
             uint4 r = make_uint4(0u, __float_as_uint(INF_F), 0u, 0u);     // weight +inf: contributes nothing
             if (i < nE) r = crec[i];
-            efr[j] = r.x & 0xFFFFu; eto[j] = r.x >> 16; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
+            eft[j] = r.x; esl[j] = r.z; ew[j] = __uint_as_float(r.y);
         }
         int c0[JS], c1[JS], em[JS];
 #pragma unroll
@@ -2297,7 +2301,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
                     const float* grow = gbase + (size_t)t * DP;
 #pragma unroll
                     for (int j = 0; j < JE; j++) {
-                        va[f][j] = load_x<SYNC>(arow + efr[j]); vb[f][j] = load_x<SYNC>(brow + eto[j]); vg[f][j] = load_x<SYNC>(grow + esl[j]);
+                        va[f][j] = load_x<SYNC>(arow + (eft[j] & 0xFFFFu)); vb[f][j] = load_x<SYNC>(brow + (eft[j] >> 16)); vg[f][j] = load_x<SYNC>(grow + esl[j]);
                     }
                 }
 #pragma unroll
@@ -2325,7 +2329,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
                 for (int j = 0; j < JE; j++) {
                     const float p = mn[f] == INF_F ? 0.f : __builtin_amdgcn_exp2f(mn[f] - x[f][j]);
                     if (NEGLOG) part[f] += p;
-                    xsb[f * COMB_BATCH_EDGES + tid + j * COMB_THREADS] = NEGLOG ? x[f][j] : p;
+                    xsb[f * XSTRIDE + tid + j * COMB_THREADS] = NEGLOG ? x[f][j] : p;
                 }
             }
             // per-emission sums in fixed (input) order and the frame normalisers
@@ -2335,7 +2339,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
 #pragma unroll
                 for (int js = 0; js < JS; js++) {
                     float s4[MF];
-                    slot_sum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], s4);
+                    slot_sum_frames<MF>(xsb, XSTRIDE, c0[js], c1[js], s4);
 #pragma unroll
                     for (int f = 0; f < MF; f++) val[f][js] = s4[f];
                 }
@@ -2356,7 +2360,7 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
 #pragma unroll
                 for (int js = 0; js < JS; js++) {
                     LogSum l4[MF];
-                    slot_logsum_frames<MF>(xsb, COMB_BATCH_EDGES, c0[js], c1[js], l4);
+                    slot_logsum_frames<MF>(xsb, XSTRIDE, c0[js], c1[js], l4);
 #pragma unroll
                     for (int f = 0; f < MF; f++)
                         val[f][js] = mn[f] == INF_F ? INF_F : neg_log_value(l4[f], mn[f], __builtin_amdgcn_logf(tot[f]));
@@ -2393,6 +2397,21 @@ __global__ __launch_bounds__(COMB_THREADS, SMALL ? COMB_SMALL_OCC : 3) void fbw_
                         if (tid + js * COMB_THREADS < D) image[(size_t)f * 4 * F4 + shf[f] + em[js]] = hole;
                 }
         }
+    };
+    bool written = false;
+    if constexpr (SMALL) {
+        if (a.batch_frames && nE <= COMB_BATCH_EDGES) {
+            batched(std::integral_constant<int, COMB_BATCH>{}, std::integral_constant<int, COMB_BATCH_EDGES / COMB_THREADS>{});
+            written = true;
+        } else if (a.batch_frames && nE <= COMB_XS) {
+            batched(std::integral_constant<int, COMB_BATCH / 2>{}, std::integral_constant<int, COMB_XS / COMB_THREADS>{});
+            written = true;
+        } else if (a.batch_frames) {
+            batched(std::integral_constant<int, 1>{}, std::integral_constant<int, COMB_BATCH * COMB_BATCH_EDGES / COMB_THREADS>{});
+            written = true;
+        }
+    }
+    if (written) {
     } else if (SMALL || (nE <= COMB_XS && D <= 2 * COMB_THREADS)) {
         // fast path: this thread's edges and slots stay in registers for the whole strip, and
         // the operands of the next frame are fetched while the current one is processed
@@ -3268,9 +3287,9 @@ size_t comb_batch_lds_bytes(int F) { return (size_t)COMB_BATCH * ((size_t)(((F +
 template <bool SYNC>
 void launch_combine(const bool neglog, const dim3 grid, const size_t lds, hipStream_t s, CombArgs ca) {
     if (!ca.direct_only && !ca.tile_w) {
-        CombArgs cs = ca;
         size_t lds_s = lds;
-        if (ca.F <= COMB_BATCH_F) { cs.batch_frames = 1; lds_s = std::max(lds, comb_batch_lds_bytes(ca.F)); }
+        if (ca.F <= COMB_BATCH_F) { ca.batch_frames = 1; lds_s = std::max(lds, comb_batch_lds_bytes(ca.F)); }      // (both instances: it decides which takes a sequence)
+        CombArgs cs = ca;
         if (neglog) hipLaunchKernelGGL((fbw_combine<SYNC, true, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
         else hipLaunchKernelGGL((fbw_combine<SYNC, false, true>), grid, dim3(COMB_THREADS), lds_s, s, cs);
         ca.small_elsewhere = 1;

@@ -178,10 +178,11 @@ def test_kernels_stay_within_their_register_budgets():
     for name, r in kernels("fbw_combine").items():
         sync, neglog, small = (int(x) for x in re.search(r"fbw_combineILb(\d)ELb(\d)ELb(\d)E", name).groups())
         if small:
-            # the instance for sequences of up to 1024 edges: six workgroups per compute unit.  Its scratch: values that
-            # do not change over a strip of frames, stored once in front of the frame loop and read back once per
-            # batch of four frames -- nothing per edge or per frame
-            assert r["vgprs"] <= 80 and r["occupancy"] >= 6 and r["scratch"] <= (72 if neglog else 40), (name, r)
+            # the instance for sequences of up to 1024 edges (2048 with short rows): six workgroups per compute unit.
+            # Its scratch: values that do not change over a strip of frames, stored once in front of the frame loop
+            # and read back once per batch of frames, and a few reloads in the sums of the variant with eight edges
+            # per thread (measured: 2.3 times faster than the general instance on such sequences all the same)
+            assert r["vgprs"] <= 80 and r["occupancy"] >= 6 and r["scratch"] <= (72 if neglog else 56), (name, r)
         elif neglog:
             # the instance for the -log output: a few reloads per frame on its paths for sequences of more than 1024
             # edges (with two waves per SIMD it needs none and is slower)

@@ -88,6 +88,8 @@ def test_tightly_constrained_alignment(oracle):
     ("cart", dict(T=300, B=3, F=12001, shuffle_edges=True)),
     ("cart", dict(T=40, B=2, F=38000, n_labels=(8, 12))),     # the largest row images that fit into LDS
     ("ctc", dict(T=40, B=8, F=50)),
+    ("ctc", dict(T=400, B=4, F=80, n_labels=(140, 190))),            # 560-940 edges, short rows: the row writer takes two frames at a time
+    ("monophone", dict(T=420, B=6, F=264, n_labels=(130, 165))),     # 1000-1240 edges, short rows: one frame, eight edges per thread
     ("ctc", dict(T=200, B=16, F=5001, shuffle_edges=True)),
     ("cart", dict(T=60, B=44, F=300, n_labels=(5, 9))),      # the largest batch whose preparation holds the gather back itself: five workgroups per sequence, a unit each
     ("cart", dict(T=60, B=45, F=300, n_labels=(5, 9))),      # one more: a one-wave kernel does it
