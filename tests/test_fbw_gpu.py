@@ -85,6 +85,8 @@ def test_tightly_constrained_alignment(oracle):
     ("monophone", {}),
     ("monophone", dict(shuffle_edges=True, seed=5)),
     ("cart", dict(T=120, B=4, F=500)),
+    ("cart", dict(T=61, B=5, F=1024, n_labels=(5, 19))),       # the longest rows the row writer takes several frames at a time
+    ("cart", dict(T=61, B=5, F=1025, n_labels=(5, 19))),       # one more float: frame by frame
     ("cart", dict(T=300, B=3, F=12001, shuffle_edges=True)),
     ("cart", dict(T=40, B=2, F=38000, n_labels=(8, 12))),     # the largest row images that fit into LDS
     ("ctc", dict(T=40, B=8, F=50)),
