@@ -191,6 +191,21 @@ def test_one_class_on_many_edges(oracle, n_labels):
     check_against_oracle(oracle, (W.am_scores, W.edges, W.weights, W.start_end_states, W.seq_lens, W.n_states), threads=8)
 
 
+@pytest.mark.parametrize("big_labels,T", [(250, 800), (500, 1550), (1150, 3500)], ids=["1500-edges", "3000-edges", "6900-edges"])
+def test_one_large_automaton_among_many_small_ones(oracle, big_labels, T):
+    """Twenty small sequences and one large one: few edges per sequence on average, so the preparation runs in
+    workgroups of 512 threads, and the large sequence's edges are sorted with four, eight and sixteen keys per thread
+    (keys in registers: partners a workgroup apart sit in the same thread)."""
+    from tests.test_flat_writer_gpu import merge
+    parts = [make_workload("cart", seed=5, T=T, B=20, F=60, n_labels=(3, 9), shuffle_edges=True),
+             make_workload("cart", seed=6, T=T, B=1, F=60, n_labels=(big_labels, big_labels))]
+    parts[1].seq_lens[:] = T
+    am, edges, weights, se, lens, n_states = merge(parts)
+    big = int((edges[3] == 20).sum())
+    assert edges.shape[1] <= 512 * 21 and big > 1024, (edges.shape, big)
+    check_against_oracle(oracle, (am, edges, weights, se, lens, n_states), threads=8)
+
+
 def test_large_batch_of_tightly_aligned_ctc(oracle):
     """More than 128 sequences (the recursion instance of which two workgroups share a compute unit) of
     CTC automata with 116 labels over up to 850 frames: float state vectors came out at 9e-5 here; the
