@@ -126,6 +126,19 @@ def test_size_classes(oracle, kind):
     assert_identical(got, oracle.viterbi_oracle(am, wl.edges, w, wl.start_end_states, wl.seq_lens, wl.n_states))
 
 
+def test_one_large_automaton_among_many_small_ones(oracle):
+    """Few edges per sequence on average (preparation in workgroups of 512 threads) and one sequence of 3000: its
+    edges are sorted with eight keys per thread; the alignment stays bit-identical."""
+    from tests.test_flat_writer_gpu import merge
+    T = 1550
+    parts = [make_workload("cart", seed=5, T=T, B=20, F=60, n_labels=(3, 9), shuffle_edges=True),
+             make_workload("cart", seed=6, T=T, B=1, F=60, n_labels=(500, 500))]
+    parts[1].seq_lens[:] = T
+    am, edges, weights, se, lens, n_states = merge(parts)
+    got = run_cabi_viterbi(-am, edges, -weights, se, lens, n_states)[:2]
+    assert_identical(got, oracle.viterbi_oracle(-am, edges, -weights, se, lens, n_states))
+
+
 def test_device_status():
     """An index out of range is reported; the sequence gets score NaN and an all-zero alignment."""
     edges = np.array([[0, 1, 1, 0], [1, 1, 9, 0]], dtype=np.int32).T.copy()      # emission class 9 of 4
